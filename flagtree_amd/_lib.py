@@ -9,6 +9,11 @@ _i32, _i64, _f32, _vp, _sz = _c.c_int32, _c.c_int64, _c.c_float, _c.c_void_p, _c
 
 SMLA_KV_BF16, SMLA_KV_FP8_B128, SMLA_KV_F32 = 0, 1, 2
 SMLA_MAX_SPLITS = 32
+SMLA_WS_COUNTER_BYTES = 262144
+SMLA_WS_HEADER_OFFSET = SMLA_WS_COUNTER_BYTES - 64
+SMLA_WS_MAGIC = 0x414C4D53
+SMLA_EWORKSPACE_STATE = -8
+WS_STATUS_BITS = {1: "never initialised", 2: "arrival word in an illegal state", 4: "split merge timed out"}
 FP8_RECORD_BYTES = 656
 
 # name -> (restype, argtypes); must list every symbol the header declares
@@ -24,6 +29,7 @@ SIGNATURES = {
     "smla_plan_splits": (_c.c_int, [_c.c_int, _i32, _i32, _i32]),
     "smla_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
     "smla_workspace_init": (_c.c_int, [_vp, _sz, _vp]),
+    "smla_workspace_status": (_c.c_int, [_vp, _sz, _vp, _c.POINTER(_c.c_uint32)]),
     "smla_gather_rows": (_c.c_int, [_vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i64,
                                     _i64, _vp]),
     "smla_merge_splits": (_c.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp]),

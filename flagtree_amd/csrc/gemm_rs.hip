@@ -289,12 +289,12 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
       const int i = 2 * wave + d;
       const uint64_t sa = (uint64_t)(uintptr_t)x + ((uint64_t)(m0 + 8 * i) * K + k0) * 2;
       const uint32_t ma = dst + i * 1024;
-      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(a_off[d & 1]), "s"(sa), "s"(ma) : "memory");
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(a_off[d & 1]), "s"(sa), "s"(ma) : "memory", "m0");
     } else {
       const int i = 2 * wave + d - 2;
       const uint64_t sb = (uint64_t)(uintptr_t)w + (uint64_t)(k0 + 2 * i) * N * 2;
       const uint32_t mb = dst + kA2Bytes + i * 1024;
-      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(b_off[d & 1]), "s"(sb), "s"(mb) : "memory");
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(b_off[d & 1]), "s"(sb), "s"(mb) : "memory", "m0");
     }
   };
 

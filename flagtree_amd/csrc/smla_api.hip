@@ -18,7 +18,8 @@ int check_common(const void* q, const void* kv, const int32_t* indices, const vo
   if (d_qk != kDqk || d_v != kDv) return SMLA_EINVAL_SHAPE;
   if (kv_rows <= 0 || kv_rows > 0x7fffffffLL || kv_seq_stride < 0) return SMLA_EINVAL_SHAPE;
   if (block_table && (page_size <= 0 || bt_stride <= 0)) return SMLA_EINVAL_SHAPE;
-  if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !aligned16(indices)) return SMLA_EINVAL_ALIGN;
+  if (!aligned16(q) || !aligned16(kv) || !aligned16(out)) return SMLA_EINVAL_ALIGN;
+  if ((reinterpret_cast<uintptr_t>(indices) & 3u) != 0) return SMLA_EINVAL_ALIGN;   // read 4 bytes at a time
   return SMLA_OK;
 }
 
@@ -49,6 +50,7 @@ const char* smla_strerror(int status) {
     case SMLA_EINVAL_SPLITS: return "n_splits out of range for this top-k length";
     case SMLA_ENODEVICE: return "no usable gfx950 device";
     case SMLA_EINVAL_SCALE: return "sm_scale must be positive and finite";
+    case SMLA_EWORKSPACE_STATE: return "a split launch flagged its workspace (uninitialised, shared by overlapping launches, or a split never arrived)";
     default: break;
   }
   if (status <= SMLA_EHIP_BASE) return hipGetErrorString((hipError_t)(SMLA_EHIP_BASE - status));
@@ -57,8 +59,8 @@ const char* smla_strerror(int status) {
 
 int smla_abi_version(void) { return 1; }
 
-// Workspace layout: [0, SMLA_WS_COUNTER_BYTES) arrival counters (zero between calls), then the
-// partial outputs [T, n_splits, H, d_v] f32 and the partial LSEs [T, n_splits, H] f32.
+// Workspace layout: [0, SMLA_WS_HEADER_OFFSET) arrival words (zero between calls), the 64-byte
+// header {magic, status, poll limit, -} up to SMLA_WS_COUNTER_BYTES, then the partial outputs [T, n_splits, H, d_v] f32 and the partial LSEs [T, n_splits, H] f32.
 size_t smla_workspace_bytes(int32_t n_tokens, int32_t n_heads, int32_t d_v, int32_t n_splits) {
   if (n_splits <= 1 || n_tokens <= 0 || n_heads <= 0 || d_v <= 0) return 0;
   return SMLA_WS_COUNTER_BYTES + (size_t)n_tokens * n_splits * n_heads * ((size_t)d_v + 1) * sizeof(float);
@@ -68,7 +70,32 @@ int smla_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
   if (!workspace) return SMLA_EINVAL_NULLPTR;
   if (!aligned16(workspace)) return SMLA_EINVAL_ALIGN;
   if (workspace_bytes < SMLA_WS_COUNTER_BYTES) return SMLA_EINVAL_WORKSPACE;
-  return launch_zero(workspace, SMLA_WS_COUNTER_BYTES, static_cast<hipStream_t>(stream));
+  return launch_workspace_init(workspace, static_cast<hipStream_t>(stream));
+}
+
+int smla_workspace_status(void* workspace, size_t workspace_bytes, void* stream, uint32_t* status_out) {
+  if (!workspace) return SMLA_EINVAL_NULLPTR;
+  if (!aligned16(workspace)) return SMLA_EINVAL_ALIGN;
+  if (workspace_bytes < SMLA_WS_COUNTER_BYTES) return SMLA_EINVAL_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint8_t* header = static_cast<uint8_t*>(workspace) + SMLA_WS_HEADER_OFFSET;
+  uint32_t h[4] = {0, 0, 0, 0};
+  hipError_t e = hipMemcpyAsync(h, header, sizeof(h), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return hip_status(e);
+  uint32_t status = h[1];
+  if (h[0] != SMLA_WS_MAGIC) status |= SMLA_WS_STATUS_UNINITIALISED;
+  if (status_out) *status_out = status;
+  if (status == 0) return SMLA_OK;
+  if (h[0] == SMLA_WS_MAGIC) {
+    // A flagged launch may have left arrival words behind (a split that arrived after the word
+    // was given up on): start over.  An uninitialised workspace stays as it is.
+    const int rc = launch_workspace_init(workspace, s);
+    if (rc != SMLA_OK) return rc;
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_status(e);
+  }
+  return SMLA_EWORKSPACE_STATE;
 }
 
 int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t topk) {
@@ -85,7 +112,7 @@ int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t t
   if (cap < 1) cap = 1;
   if (want > cap) want = cap;
   if (want > SMLA_MAX_SPLITS) want = SMLA_MAX_SPLITS;
-  if (groups * 8 > SMLA_WS_COUNTER_BYTES) want = 1;        // more (token, head block) pairs than counters
+  if (groups * 8 > SMLA_WS_HEADER_OFFSET) want = 1;        // more (token, head block) pairs than arrival words
   return want < 1 ? 1 : want;
 }
 
@@ -95,6 +122,7 @@ static int fill_params(Params& p, const void* q, const void* kv, const int32_t* 
                        int32_t bt_stride, int64_t kv_seq_stride, int64_t kv_rows, float sm_scale) {
   p.q = q; p.kv = kv; p.indices = indices; p.seq_lens = nullptr; p.block_table = block_table; p.out = out; p.lse = lse;
   p.part_out = nullptr; p.part_lse = nullptr; p.counters = nullptr;
+  p.ws_header = static_cast<uint32_t*>(const_cast<void*>(q));   // (read, never used, when nothing is split)
   p.n_tokens = n_tokens; p.tokens_per_seq = tokens_per_seq; p.n_heads = n_heads; p.topk = topk;
   p.page_size = block_table ? page_size : 1; p.bt_stride = block_table ? bt_stride : 0;
   p.n_splits = 1; p.split_len = topk;
@@ -138,8 +166,9 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
   if (n_splits > 1) {
     const size_t need = smla_workspace_bytes(n_tokens, n_heads, d_v, n_splits);
     if (!workspace || workspace_bytes < need || !aligned16(workspace)) return SMLA_EINVAL_WORKSPACE;
-    if ((size_t)n_tokens * ((n_heads + 15) / 16) * 8 > SMLA_WS_COUNTER_BYTES) return SMLA_EINVAL_SPLITS;
+    if ((size_t)n_tokens * ((n_heads + 15) / 16) * 8 > SMLA_WS_HEADER_OFFSET) return SMLA_EINVAL_SPLITS;
     p.counters = static_cast<unsigned long long*>(workspace);
+    p.ws_header = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(workspace) + SMLA_WS_HEADER_OFFSET);
     p.part_out = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + SMLA_WS_COUNTER_BYTES);
     p.part_lse = p.part_out + (size_t)n_tokens * n_splits * n_heads * d_v;
   }

@@ -27,6 +27,7 @@ struct Params {
   float* part_out;   // [T, n_splits, H, d_v] when n_splits > 1
   float* part_lse;   // [T, n_splits, H]
   unsigned long long* counters; // [T, ceil(H/64)] arrival tickets + published bits, zero between calls
+  uint32_t* ws_header;          // workspace header {magic, status, spin limit, -}; any readable word when n_splits == 1
   int32_t n_tokens, tokens_per_seq, n_heads, topk;
   int32_t page_size, bt_stride, n_splits, split_len;
   int64_t kv_seq_stride, kv_rows;
@@ -78,6 +79,71 @@ __device__ __forceinline__ void translate_entries4(const Params& p, int seq, int
 #pragma unroll
     for (int k = 0; k < 4; ++k) rr[k] = translate_unpaged(p, seq, rr[k]);
   }
+}
+
+// ---- split merge inside a launch: arrival protocol ------------------------------------------
+// Every (token, head block) owns one 64-bit word of the workspace: high half = arrival tickets,
+// low half = one "partial published" bit per split.  The word is zero between launches.  A word
+// that is not (a workspace that never went through smla_workspace_init, two launches sharing a
+// workspace at the same time) must neither hang the launch nor pass for a result: the header of
+// the workspace carries a magic word, a status word the host can read back, and the number of
+// polls the last arrival may spend waiting for the others.
+constexpr uint32_t kWsMagic = SMLA_WS_MAGIC;
+enum { kRolePublish = 0, kRoleLast = 1, kRoleError = 2 };
+
+typedef __attribute__((ext_vector_type(4))) uint32_t ws_u32x4;
+
+__device__ __forceinline__ void ws_flag(const Params& p, uint32_t bits) {
+  __hip_atomic_fetch_or(p.ws_header + 1, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One thread of the workgroup: take an arrival ticket and decide the workgroup's role.  `magic`
+// is the header's first word as read at kernel entry.  An inconsistent word (more arrivals than
+// splits, my own bit or a bit past the last split already set, more published than arrived)
+// flags the workspace and zeroes the word (the host re-initialises a flagged workspace: a split
+// that arrives after this may leave its ticket behind).
+__device__ __forceinline__ int ws_arrive(const Params& p, unsigned long long* word, uint32_t magic, int ns, int sp) {
+  if (magic != kWsMagic) {
+    ws_flag(p, SMLA_WS_STATUS_UNINITIALISED);
+    return kRoleError;
+  }
+  const unsigned long long old = __hip_atomic_fetch_add(word, 1ull << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint32_t ticket = (uint32_t)(old >> 32), bits = (uint32_t)old;
+  const uint32_t legal = ns >= 32 ? 0xffffffffu : (1u << ns) - 1u;
+  if (ticket >= (uint32_t)ns || (bits & ~legal) != 0 || (bits & (1u << sp)) != 0 || (uint32_t)__popc(bits) > ticket) {
+    ws_flag(p, SMLA_WS_STATUS_STALE);
+    __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return kRoleError;
+  }
+  return ticket == (uint32_t)ns - 1 ? kRoleLast : kRolePublish;
+}
+
+// One thread of the last workgroup to arrive: poll until every other split has published, at
+// most `spin limit` times (the others hold tickets, so they are past their loops and publish
+// within microseconds; the limit is what ends the wait when the word was not what it seemed).
+// Gives up by flagging the workspace and zeroing the word.
+__device__ __forceinline__ bool ws_wait_published(const Params& p, unsigned long long* word, int ns, int sp) {
+  const unsigned long long legal = ns >= 32 ? 0xffffffffull : (1ull << ns) - 1ull;
+  const unsigned long long others = legal & ~(1ull << sp);
+  const uint32_t limit = __hip_atomic_load(p.ws_header + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (uint32_t n = 0; n < limit; ++n) {
+    if ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & others) == others) return true;
+    __builtin_amdgcn_s_sleep(2);
+  }
+  ws_flag(p, SMLA_WS_STATUS_TIMEOUT);
+  __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return false;
+}
+
+// Partials cross workgroups without fences: stored and loaded at agent scope (sc1: through the
+// L2, past the per-CU cache), a bit is published only after the stores have been acknowledged.
+// The loads are buffer loads the compiler can see: it counts them in flight and waits where a
+// landing register is first read, whatever copies or spills it puts in between.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t ws_partial_rsrc(const float* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ ws_u32x4 ws_load_partial(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 16 /* sc1 */);
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
@@ -132,6 +198,7 @@ int launch_kv_copy(const void* src, const int64_t* slot, void* pool, int64_t n_r
 int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_t* out, int n_rows,
                         int n_cols, long long row_stride, int k, hipStream_t s);
 int launch_zero(void* ptr, size_t bytes, hipStream_t s);
+int launch_workspace_init(void* workspace, hipStream_t s);
 int launch_gemm_rs(const void* x, const void* w, const float* partial, void* out, int m, int n,
                    int k, int n_chunks, int64_t chunk_stride, hipStream_t s);
 

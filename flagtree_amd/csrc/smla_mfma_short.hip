@@ -2,14 +2,16 @@
 // e.g. one GPU's 16-head slice of a 128-head model over an fp8 KV cache.
 //
 // One workgroup of 4 wavefronts handles (token, block of 16 heads, split of the top-k list).
-// 64-token tiles of raw KV rows (bf16 rows or 656-byte fp8 records) stream global -> LDS
-// through direct-to-LDS loads into a two-deep ring: nothing but bytes in flight, no registers.
-// Wavefront w owns tokens 16w .. 16w+15 of every tile and is otherwise independent of its
+// Wavefront w owns tokens 16w .. 16w+15 of every 64-token tile and is otherwise independent of its
 // siblings: it has its own softmax reference, row sums and [16 heads x 512] accumulator, which
-// are merged once at the end.  Per tile a wavefront
-//   * (fp8 only) dequantises its 16 records in registers into a private bf16 staging area in LDS:
-//     the e4m3 values are converted exactly, the per-128-block fp32 scales multiply the per-block
-//     partial scores and the probabilities (all in fp32),
+// are merged once at the end.
+//   * bf16 rows stream global -> LDS through direct-to-LDS loads into a two-deep ring shared by
+//     the workgroup (one barrier per tile).
+//   * fp8 records stream through registers, every wavefront its own 16 records of a tile, two
+//     tiles in flight; a landed tile is dequantised into the wavefront's private bf16 staging
+//     area in LDS: the e4m3 values are converted exactly, the per-128-block fp32 scales multiply
+//     the per-block partial scores and the probabilities (all in fp32).  No barrier in the loop.
+// Per tile a wavefront computes
 //   * S^T[16 tok x 16 heads] = K[16 x 576] . Q^T[576 x 16]   v_mfma_f32_16x16x32_bf16, Q in VGPRs
 //   * probabilities per head (lane = head), kept as the A operand of the next product
 //   * O[16 heads x 512] += P[16 x 16 tok] . V[16 tok x 512]    v_mfma_f32_16x16x16_bf16, B through
@@ -61,12 +63,6 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-// Direct-to-LDS gather of one tile: wave-wide 16-byte loads, the wave's 64 chunks land in 1 KB
-// of consecutive LDS at M0.  Rows past the valid count repeat the last valid row (masked later).
-// bf16: tile = 64 rows x 73 slots (72 data + 1 pad) = 73 wave loads over a linear slot space; a
-// lane on a pad slot re-reads the row's last chunk.
-// fp8: one load per 656-byte record (41 active lanes) with a scalar row base, so issuing a tile
-// costs scalar instructions only; records stay unpadded (they are only ever read 16 B at a time).
 // bf16: direct-to-LDS gather of one tile: wave-wide 16-byte loads, the wave's 64 chunks land in 1 KB
 // of consecutive LDS at M0; tile = 64 rows x 73 slots (72 data + 1 pad) = 73 wave loads over a
 // linear slot space; a lane on a pad slot re-reads the row's last chunk.  Rows past the valid count
@@ -89,7 +85,7 @@ __device__ __forceinline__ void dma_tile_bf16(const uint8_t* kv, const int32_t* 
     const uint8_t* src = kv + (size_t)r[i] * kRowBytesBf16 + col * 16;
     const uint32_t m0v = __builtin_amdgcn_readfirstlane(tile_lds + (4 * i + wave) * 1024);
     if (4 * i + 3 < kLoads || 4 * i + wave < kLoads) {           // wave-uniform
-      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(m0v) : "memory");
+      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(m0v) : "memory", "m0");
     }
   }
 }
@@ -182,6 +178,7 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
   const int head = head0 + l16;
   const bool head_ok = head < p.n_heads;
   const uint8_t* kv = static_cast<const uint8_t*>(p.kv);
+  const uint32_t ws_magic = *p.ws_header;    // read long before the split merge needs it
 
   // ---- the first chunk's index loads go out before anything else: the row list they lead to
   // (index -> page table -> row fetch) is the longest dependent chain of the kernel
@@ -467,14 +464,19 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
   }
 
   // ---- split merge inside the launch (ticket word per (token, head block): high half arrival
-  // count, low half one "published" bit per split; partials move with agent-scope accesses).
+  // count, low half one "published" bit per split; partials move with agent-scope accesses; an
+  // illegal word or a wait past the workspace's poll limit flags the workspace and marks the
+  // rows' LSE with NaN, see ws_arrive / ws_wait_published).
   const int ns = p.n_splits;
   unsigned long long* word = p.counters + (size_t)t * n_hblocks + hb;
-  if (tid == 0)
-    s_nvalid = (int)(__hip_atomic_fetch_add(word, 1ull << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+  if (tid == 0) s_nvalid = ws_arrive(p, word, ws_magic, ns, sp);
   __syncthreads();
-  const bool last = s_nvalid == ns - 1;
-  if (!last) {
+  const int role = s_nvalid;
+  auto give_up = [&]() {                     // the workspace was not what it should be: mark the rows
+    if (wave == 0 && q4 == 0 && head_ok) p.lse[(size_t)t * p.n_heads + head] = __uint_as_float(0x7fc00000u);
+  };
+  if (role == kRoleError) { give_up(); return; }
+  if (role == kRolePublish) {
     if (wave == 0 && q4 == 0 && head_ok)
       __hip_atomic_store(&p.part_lse[((size_t)t * ns + sp) * p.n_heads + head], lse_nat, __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
@@ -496,12 +498,9 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
   // all of them, then fold the normalised partials in split order with every product and sum
   // rounded on its own (no fused multiply-add): the result does not depend on which split
   // happened to arrive last.  Per-head scalars live in lane = head l16 of every wavefront.
-  if (tid == 0) {
-    const unsigned long long others = ((ns >= 32 ? 0xffffffffull : (1ull << ns) - 1ull)) & ~(1ull << sp);
-    while ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & others) != others)
-      __builtin_amdgcn_s_sleep(2);
-  }
+  if (tid == 0) s_flag = ws_wait_published(p, word, ns, sp) ? 0 : 1;
   __syncthreads();
+  if (s_flag != 0) { give_up(); return; }
   auto split_lse = [&](int i) {
     if (i == sp) return lse_nat;
     return head_ok ? __hip_atomic_load(&p.part_lse[((size_t)t * ns + i) * p.n_heads + head], __ATOMIC_RELAXED,
@@ -531,11 +530,10 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
         v[j] = f32x4{a4.x, a4.y, a4.z, a4.w};
       }
     } else {
-      const float* src = p.part_out + (((size_t)t * ns + i) * p.n_heads + min(head0 + orow, p.n_heads - 1)) * kDv + ocol;
+      const __amdgpu_buffer_rsrc_t src = ws_partial_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0) * kDv);
+      const uint32_t off = (uint32_t)((min(orow, p.n_heads - 1 - head0) * kDv + ocol) * 4);
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[j]) : "v"(src + 64 * j) : "memory");
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      for (int j = 0; j < 8; ++j) v[j] = __builtin_bit_cast(f32x4, ws_load_partial(src, off + 256 * j));
     }
     const float rb = s_f[wave][orow];
 #pragma unroll

@@ -105,7 +105,7 @@ struct DmaTile {
       const uint64_t sbase = (uint64_t)(uintptr_t)kv + (uint64_t)srow * kRowBytesBf16;
       const uint32_t m0v = tile_lds + r * kMainStride;
       const uint32_t vsw = voff ^ (uint32_t)(swz(r) << 4);
-      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(vsw), "s"(sbase), "s"(m0v) : "memory");
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(vsw), "s"(sbase), "s"(m0v) : "memory", "m0");
     } else {
       // lane l fills slot l of the 1 KB block of pairs 4*wave .. 4*wave+3
       const int pair = 4 * wave + (lane >> 4);
@@ -113,7 +113,7 @@ struct DmaTile {
       const int32_t trow = __shfl(rid, r);
       const uint8_t* src = kv + (size_t)trow * kRowBytesBf16 + 1024 + c * 16;
       const uint32_t m0v = tile_lds + kRopeBase + wave * 1024;
-      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(m0v) : "memory");
+      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(m0v) : "memory", "m0");
     }
   }
 };
@@ -329,6 +329,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   const bool head_ok = head < p.n_heads;
   const uint8_t* kv = static_cast<const uint8_t*>(p.kv);
   const int k_begin = sp * p.split_len, k_end = min(k_begin + p.split_len, p.topk);
+  const uint32_t ws_magic = *p.ws_header;    // read long before the split merge needs it
 
   // ---- the first chunk's index loads go out before anything else: the row list they lead to
   // (index -> page table -> row fetch) is the longest dependent chain of the kernel
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
       const int e = 256 * c + 4 * lane;
       const uint32_t m0v = lds_bt + 1024 * c;
       if (e < p.bt_stride)
-        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(bt_row + e), "s"(m0v) : "memory");
+        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(bt_row + e), "s"(m0v) : "memory", "m0");
     }
   }
 
@@ -557,7 +558,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
             const int e = min((it + kSlots) * kTN + (tid >> 3), n_valid - 1);
             const uint8_t* line = kv + (size_t)s_rows[e] * kRowBytesFp8 + min((tid & 7) * 128, kRowBytesFp8 - 4);
             const uint32_t sink = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)&s_sink[0];
-            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(line), "s"(sink) : "memory");
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(line), "s"(sink) : "memory", "m0");
           }
         }
         // Tile it+1 is never the last one here, so it is full: no masking, and the reference is
@@ -644,8 +645,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // the arrival ticket of the split merge is taken here, so that its round trip to memory
   // overlaps the staging below (the merge itself is described further down)
   if (p.n_splits > 1 && tid == 0)
-    s_nvalid = (int)(__hip_atomic_fetch_add(p.counters + (size_t)t * n_hblocks + hb, 1ull << 32, __ATOMIC_RELAXED,
-                                            __HIP_MEMORY_SCOPE_AGENT) >> 32);
+    s_nvalid = ws_arrive(p, p.counters + (size_t)t * n_hblocks + hb, ws_magic, p.n_splits, sp);
 #pragma unroll
   for (int ht = 0; ht < 2; ++ht) {
     float l = l_part[ht];
@@ -696,11 +696,17 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // Partials move between workgroups without fences: they are stored and loaded with the
   // sc1 (agent scope: write-through / read-through the L2) modifier, and a bit is published
   // only after the stores have been acknowledged.  A release / acquire fence pair would write
-  // back and invalidate the whole L2 of the XCD instead.
+  // back and invalidate the whole L2 of the XCD instead.  A word that is not in a legal state,
+  // or a wait that outlasts the workspace's poll limit, flags the workspace, marks the rows'
+  // LSE with NaN and leaves (see ws_arrive / ws_wait_published).
   const int ns = p.n_splits;
   unsigned long long* word = p.counters + (size_t)t * n_hblocks + hb;
-  const bool last = s_nvalid == ns - 1;                            // ticket taken at the top of the epilogue
-  if (!last) {
+  const int role = s_nvalid;                                       // ticket taken at the top of the epilogue
+  auto give_up = [&]() {                                           // the workspace was not what it should be: mark the rows
+    if (dh == 0 && g == 0 && head_ok) p.lse[(size_t)t * p.n_heads + head] = __uint_as_float(0x7fc00000u);
+  };
+  if (role == kRoleError) { give_up(); return; }
+  if (role == kRolePublish) {
     if (dh == 0 && g == 0 && head_ok)
       __hip_atomic_store(&p.part_lse[((size_t)t * ns + sp) * p.n_heads + head], lse_nat, __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
@@ -720,12 +726,9 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // all of them, then fold the normalised partials in split order with every product and sum
   // rounded on its own (no fused multiply-add): the result does not depend on which split
   // happened to arrive last.  Per-head scalars live in lane = head row c32.
-  if (tid == 0) {
-    const unsigned long long others = ((ns >= 32 ? 0xffffffffull : (1ull << ns) - 1ull)) & ~(1ull << sp);
-    while ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & others) != others)
-      __builtin_amdgcn_s_sleep(2);
-  }
+  if (tid == 0) s_redo = ws_wait_published(p, word, ns, sp) ? 0 : 1;
   __syncthreads();
+  if (s_redo != 0) { give_up(); return; }
   auto split_lse = [&](int i) {
     if (i == sp) return lse_nat;
     return head_ok ? __hip_atomic_load(&p.part_lse[((size_t)t * ns + i) * p.n_heads + head], __ATOMIC_RELAXED,
@@ -766,11 +769,10 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
           v[j] = f32x4{a4.x, a4.y, a4.z, a4.w};
         }
       } else {
-        const float* src = p.part_out + (((size_t)t * ns + i) * p.n_heads + head0) * kDv + col4;
+        const __amdgpu_buffer_rsrc_t src = ws_partial_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0) * kDv);
 #pragma unroll
         for (int j = 0; j < 16; ++j)
-          asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[j]) : "v"(src + (size_t)min(r0 + j, n_rows - 1) * kDv) : "memory");
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          v[j] = __builtin_bit_cast(f32x4, ws_load_partial(src, (uint32_t)((min(r0 + j, n_rows - 1) * kDv + col4) * 4)));
       }
 #pragma unroll
       for (int j = 0; j < 16; ++j) {

@@ -358,4 +358,16 @@ int launch_zero(void* ptr, size_t bytes, hipStream_t s) {
   return hip_status(hipGetLastError());
 }
 
+// zeroes the arrival words of a workspace and writes its header (same reason for a kernel)
+__global__ __launch_bounds__(256) void workspace_init_kernel(uint4* __restrict__ p) {
+  constexpr size_t kWords16 = SMLA_WS_COUNTER_BYTES / 16, kHeader16 = SMLA_WS_HEADER_OFFSET / 16;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < kWords16; i += (size_t)gridDim.x * 256)
+    p[i] = i == kHeader16 ? make_uint4(SMLA_WS_MAGIC, 0u, SMLA_WS_SPIN_LIMIT_DEFAULT, 0u) : make_uint4(0, 0, 0, 0);
+}
+
+int launch_workspace_init(void* workspace, hipStream_t s) {
+  workspace_init_kernel<<<dim3(64), dim3(256), 0, s>>>(static_cast<uint4*>(workspace));
+  return hip_status(hipGetLastError());
+}
+
 }  // namespace smla

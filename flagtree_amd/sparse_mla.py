@@ -22,9 +22,23 @@ def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-def _normalise(q, kv_cache, indices, d_v, block_table, kv_format):
+_I32_MAX = 2 ** 31 - 1
+
+
+def _indices_i32(idx2):
+    """int64 -> int32 without wrapping: anything past int32 is past every cache (at most 2^31 - 1
+    rows), so it is clamped to a value the kernels mask; negatives stay negative."""
+    if idx2.dtype == torch.int32:
+        return idx2
+    return idx2.clamp(min=-1, max=_I32_MAX).to(torch.int32)
+
+
+def _normalise(q, kv_cache, indices, d_v, block_table, kv_format, per_sequence=None):
     """Shape / dtype validation shared by the MFMA and scalar entry points.
-    Returns (q3, kv2, idx2, B, S, H, K, fmt, kv_seq_stride, block_table, out_shape, lse_shape)."""
+    Returns (q3, kv2, idx2, B, S, H, K, fmt, kv_seq_stride, block_table, out_shape, lse_shape).
+    ``per_sequence`` (only without a block table): True = kv_cache[b] is sequence b's own rows and
+    indices address them, False = one shared pool addressed by row number, None = per-sequence
+    exactly when kv_cache has a leading dim equal to the batch and the batch is larger than 1."""
     if q.dim() == 4:
         B, S, H, D = q.shape
     elif q.dim() == 3:
@@ -65,17 +79,23 @@ def _normalise(q, kv_cache, indices, d_v, block_table, kv_format):
     for name, t in (("q", q), ("kv_cache", kv_cache), ("indices", indices)):
         if not t.is_cuda:
             raise ValueError(f"{name} must be a device tensor (there is no CPU path)")
-    idx2 = indices.reshape(T, K)
-    if idx2.dtype != torch.int32:
-        idx2 = idx2.to(torch.int32)
+    idx2 = _indices_i32(indices.reshape(T, K))
     if not idx2.is_contiguous():
         idx2 = idx2.contiguous()
     q3 = q.reshape(T, H, D)
     if not q3.is_contiguous():
         q3 = q3.contiguous()
     kv_seq_stride = 0
-    if block_table is None and kv_cache.dim() >= 3 and kv_cache.shape[0] == B and B > 1:
-        kv_seq_stride = kv_cache[0].numel() // kv_cache.shape[-1]      # rows per sequence
+    if block_table is not None:
+        if per_sequence:
+            raise ValueError("per_sequence addressing and a block table exclude each other")
+    else:
+        if per_sequence is None:
+            per_sequence = kv_cache.dim() >= 3 and kv_cache.shape[0] == B and B > 1
+        if per_sequence:
+            if kv_cache.dim() < 3 or kv_cache.shape[0] != B:
+                raise ValueError("per_sequence=True needs kv_cache [B, rows per sequence, ..., D]")
+            kv_seq_stride = kv_cache[0].numel() // kv_cache.shape[-1]      # rows per sequence
     kv2 = kv_cache.reshape(-1, kv_cache.shape[-1])
     if not kv2.is_contiguous():
         kv2 = kv2.contiguous()
@@ -90,23 +110,65 @@ def _normalise(q, kv_cache, indices, d_v, block_table, kv_format):
     return q3, kv2, idx2, B, S, H, K, fmt, kv_seq_stride, block_table, out_shape, lse_shape
 
 
-_workspaces = {}    # device -> initialised workspace tensor (grown on demand)
+_workspaces = {}    # (device, stream) -> initialised workspace tensor (grown on demand)
 
 
 def make_workspace(n_bytes, device):
-    """Allocate a split workspace and zero its arrival counters (needed once per allocation)."""
-    ws = torch.empty(max(int(n_bytes), 1 << 18), dtype=torch.uint8, device=device)
+    """Allocate a split workspace, zero its arrival words and write its header (once per allocation).
+    Calls that share a workspace must not overlap: give every stream its own."""
+    ws = torch.empty(max(int(n_bytes), _lib.SMLA_WS_COUNTER_BYTES), dtype=torch.uint8, device=device)
     rc = _lib.load().smla_workspace_init(ws.data_ptr(), ws.numel(), _stream(ws))
     _lib.check(rc, "smla_workspace_init")
     return ws
 
 
+def workspace_status(workspace):
+    """Wait for the current stream and report what the split launches left in ``workspace``'s header.
+    Returns 0 when healthy; otherwise raises RuntimeError naming the SMLA_WS_STATUS bits, after the
+    library has initialised the workspace again."""
+    _check_workspace(workspace, 0, workspace.device)
+    import ctypes
+    status = ctypes.c_uint32(0)
+    rc = _lib.load().smla_workspace_status(workspace.data_ptr(), workspace.numel(), _stream(workspace),
+                                           ctypes.byref(status))
+    if rc == _lib.SMLA_EWORKSPACE_STATE:
+        what = ", ".join(name for bit, name in _lib.WS_STATUS_BITS.items() if status.value & bit)
+        raise RuntimeError(f"split workspace flagged by a launch: {what} (status {status.value})")
+    _lib.check(rc, "smla_workspace_status")
+    return 0
+
+
+def _check_workspace(workspace, need, device):
+    if not isinstance(workspace, torch.Tensor) or not workspace.is_cuda or workspace.device != device:
+        raise ValueError("workspace must be a tensor on the inputs' device (see make_workspace)")
+    if workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+        raise ValueError("workspace must be a contiguous uint8 tensor (see make_workspace)")
+    if workspace.numel() < max(need, _lib.SMLA_WS_COUNTER_BYTES):
+        raise ValueError(f"workspace too small: {max(need, _lib.SMLA_WS_COUNTER_BYTES)} bytes needed (see make_workspace)")
+
+
 def _default_workspace(n_bytes, device):
-    ws = _workspaces.get(device)
+    # One workspace per (device, stream): launches on one stream run in order, so they may share
+    # the arrival words and partials; launches on different streams may overlap and must not.
+    # A workspace that has to grow is replaced; the old tensor goes back to torch's allocator,
+    # which keeps it away from other streams until this stream's queued work is done.
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < n_bytes:
         ws = make_workspace(n_bytes, device)
-        _workspaces[device] = ws
+        _workspaces[key] = ws
     return ws
+
+
+def _resolve_workspace(workspace, ws_bytes, device):
+    """(pointer, size) of the workspace a split launch uses: the caller's (validated) or the stream's own."""
+    if not ws_bytes:
+        return None, 0
+    if workspace is None:
+        workspace = _default_workspace(ws_bytes, device)
+    else:
+        _check_workspace(workspace, ws_bytes, device)
+    return workspace.data_ptr(), workspace.numel()
 
 
 def plan_splits(n_tokens, n_heads, topk, kv_format="bf16"):
@@ -115,7 +177,7 @@ def plan_splits(n_tokens, n_heads, topk, kv_format="bf16"):
 
 
 def sparse_mla_fwd(q, kv_cache, indices, sm_scale=None, d_v=D_V, *, block_table=None, page_size=64,
-                   kv_format=None, n_splits=None, lse_base2=False, workspace=None):
+                   kv_format=None, n_splits=None, lse_base2=False, workspace=None, per_sequence=None):
     """Sparse MLA forward: attend each query token to its top-k latent KV rows.
 
     q         [B, S, H, 576] (or [T, H, 576]) bf16; fp32 for the fp32 plumbing format
@@ -123,12 +185,16 @@ def sparse_mla_fwd(q, kv_cache, indices, sm_scale=None, d_v=D_V, *, block_table=
               are flattened: [pages, page_size, 576], [B, S_kv, 1, 576], [N, 576] ...
     indices   [B, S, topk] int32; -1 = padding.  With ``block_table`` [B, max_pages] they are
               logical positions translated through the table (page_size tokens per page);
-              without it they address kv_cache rows of the token's own sequence when
-              kv_cache has a leading batch dim, else rows of the shared pool.
+              without it they address kv_cache rows of the token's own sequence
+              (``per_sequence=True``; the default when kv_cache has a leading batch dim and
+              B > 1) or rows of one shared pool (``per_sequence=False``).  int64 is accepted;
+              values past int32 are masked like any index past the cache.
+    workspace only for split launches: a tensor from ``make_workspace``; default = one per
+              (device, stream), since launches that share a workspace must not overlap.
     Returns (out [B, S, H, 512] in q's dtype, lse [B, S, H] fp32, natural log unless lse_base2).
     """
     q3, kv2, idx2, B, S, H, K, fmt, kv_seq_stride, block_table, out_shape, lse_shape = _normalise(
-        q, kv_cache, indices, d_v, block_table, kv_format)
+        q, kv_cache, indices, d_v, block_table, kv_format, per_sequence)
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D_QK)
     lib = _lib.load()
@@ -140,14 +206,7 @@ def sparse_mla_fwd(q, kv_cache, indices, sm_scale=None, d_v=D_V, *, block_table=
         raise ValueError(f"n_splits must be in [1, {_lib.SMLA_MAX_SPLITS}]")
     eff = ns if ns else lib.smla_plan_splits(fmt, T, H, K)
     ws_bytes = lib.smla_workspace_bytes(T, H, D_V, eff)
-    ws_ptr = None
-    if ws_bytes:
-        if workspace is None:
-            workspace = _default_workspace(ws_bytes, q.device)      # shared per device: calls must not overlap
-        elif workspace.numel() * workspace.element_size() < ws_bytes:
-            raise ValueError(f"workspace too small: {ws_bytes} bytes needed (see make_workspace)")
-        ws_ptr = workspace.data_ptr()
-        ws_bytes = workspace.numel() * workspace.element_size()
+    ws_ptr, ws_bytes = _resolve_workspace(workspace, ws_bytes, q.device)
     rc = lib.smla_fwd(fmt, q3.data_ptr(), kv2.data_ptr(), idx2.data_ptr(),
                       block_table.data_ptr() if block_table is not None else None,
                       out.data_ptr(), lse.data_ptr(), T, S, H, K, D_QK, D_V, page_size,
@@ -160,10 +219,10 @@ def sparse_mla_fwd(q, kv_cache, indices, sm_scale=None, d_v=D_V, *, block_table=
 
 
 def sparse_mla_fwd_scalar(q, kv_cache, indices, sm_scale=None, d_v=D_V, *, block_table=None,
-                          page_size=64, kv_format=None):
+                          page_size=64, kv_format=None, per_sequence=None):
     """Same operator on the exact-fp32 scalar device kernel (slow; cross-check for the MFMA path)."""
     q3, kv2, idx2, B, S, H, K, fmt, kv_seq_stride, block_table, out_shape, lse_shape = _normalise(
-        q, kv_cache, indices, d_v, block_table, kv_format)
+        q, kv_cache, indices, d_v, block_table, kv_format, per_sequence)
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D_QK)
     lib = _lib.load()
@@ -187,13 +246,17 @@ def gather_rows(kv_cache, indices, *, block_table=None, page_size=64, tokens_per
     if not kv_cache.is_cuda or not indices.is_cuda:
         raise ValueError("gather_rows needs device tensors (there is no CPU path)")
     kv2 = kv_cache.reshape(-1, kv_cache.shape[-1]).contiguous()
-    idx2 = indices.reshape(-1, indices.shape[-1]).to(torch.int32).contiguous()
+    if indices.dtype not in (torch.int32, torch.int64):
+        raise ValueError("indices must be int32 or int64")
+    idx2 = _indices_i32(indices.reshape(-1, indices.shape[-1])).contiguous()
     T, K = idx2.shape
     row_bytes = kv2.shape[1] * kv2.element_size()
     phys = torch.empty((T, K), dtype=torch.int32, device=kv2.device)
     rows = torch.empty((T, K, kv2.shape[1]), dtype=kv2.dtype, device=kv2.device) if with_rows else None
     if block_table is not None:
-        block_table = block_table.to(torch.int32).contiguous()
+        if block_table.dtype != torch.int32 or not block_table.is_cuda:
+            raise ValueError("block_table must be an int32 device tensor")
+        block_table = block_table.contiguous()
     lib = _lib.load()
     rc = lib.smla_gather_rows(kv2.data_ptr(), row_bytes, idx2.data_ptr(),
                               block_table.data_ptr() if block_table is not None else None,
@@ -306,7 +369,7 @@ def topk_indices(scores, k, context_lens=None):
 
 
 def decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len, attn_logits=None, num_kv_splits=None,
-                         sm_scale=None, page_size=1, logit_cap=0.0, *, kv_format=None, workspace=None):
+                         sm_scale=None, page_size=1, logit_cap=0.0, en_wmma=True, *, kv_format=None, workspace=None):
     """Dense MLA decode over the whole paged context of every sequence (no index list).
 
     Mirrors the reference's ``decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len,
@@ -320,7 +383,10 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len, attn
       o            [B, H, 512] output in q's dtype, written in place (None = allocate)
       req_to_token [B, max_pages] int32 page numbers: position p of sequence b lives in cache row
                    ``req_to_token[b, p // page_size] * page_size + p % page_size`` (reference :278-283)
-      b_seq_len    [B] int32 context lengths
+      b_seq_len    [B] int32 context lengths; a length past ``max_pages * page_size`` attends to
+                   the positions the table covers
+      en_wmma      the reference's switch between its matrix-core and plain kernels; accepted and
+                   ignored (there is one kernel)
       attn_logits  the reference's split scratch [B, H, splits, 513]; accepted and ignored (the
                    library's own workspace holds the split partials)
       logit_cap    must be 0 (the tanh cap of the reference is not implemented)
@@ -332,7 +398,10 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len, attn
     for name, t in (("q", q), ("k_buffer", k_buffer), ("req_to_token", req_to_token), ("b_seq_len", b_seq_len)):
         if not t.is_cuda:
             raise ValueError(f"{name} must be a device tensor (there is no CPU path)")
-    if v_buffer is not None and (v_buffer.data_ptr() != k_buffer.data_ptr() or v_buffer.shape[-1] != D_V):
+    if v_buffer is not None and (v_buffer.data_ptr() != k_buffer.data_ptr() or v_buffer.shape[-1] != D_V or
+                                 v_buffer.dtype != k_buffer.dtype or v_buffer.dim() != k_buffer.dim() or
+                                 tuple(v_buffer.shape[:-1]) != tuple(k_buffer.shape[:-1]) or
+                                 v_buffer.stride() != k_buffer.stride()):
         raise ValueError("v_buffer must be k_buffer[..., :512]: the latent cache holds keys and values in one row")
     B, H, _ = q.shape
     if kv_format is None:
@@ -365,14 +434,7 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len, attn
         raise ValueError(f"num_kv_splits must be in [1, {_lib.SMLA_MAX_SPLITS}]")
     eff = ns if ns else lib.smla_plan_splits(fmt, B, H, max_len)
     ws_bytes = lib.smla_workspace_bytes(B, H, D_V, eff)
-    ws_ptr = None
-    if ws_bytes:
-        if workspace is None:
-            workspace = _default_workspace(ws_bytes, q.device)
-        elif workspace.numel() * workspace.element_size() < ws_bytes:
-            raise ValueError(f"workspace too small: {ws_bytes} bytes needed (see make_workspace)")
-        ws_ptr = workspace.data_ptr()
-        ws_bytes = workspace.numel() * workspace.element_size()
+    ws_ptr, ws_bytes = _resolve_workspace(workspace, ws_bytes, q.device)
     q3 = q.contiguous()
     kv_rows = k_buffer.numel() // row
     rc = lib.smla_decode_dense(fmt, q3.data_ptr(), k_buffer.data_ptr(), seq.data_ptr(), bt.data_ptr(), o.data_ptr(),

@@ -3,7 +3,8 @@
  *
  * Plain pointers and sizes only.  Every pointer named "device" must be HIP device
  * memory of the current device; `stream` is a hipStream_t passed as void* (NULL =
- * the default stream).  All launches are asynchronous on `stream`.  The library
+ * the default stream).  All launches are asynchronous on `stream`.  q, kv, out, workspaces and
+ * the GEMM operands must be 16-byte aligned, index lists and sequence lengths 4-byte aligned.  The library
  * never allocates or frees device memory and keeps no state between calls.
  * Functions return SMLA_OK (0) or a negative error code; they never abort.
  *
@@ -34,6 +35,7 @@ enum {
   SMLA_EINVAL_SPLITS = -5,    /* n_splits outside [1, SMLA_MAX_SPLITS] */
   SMLA_ENODEVICE = -6,        /* no gfx950 device / kernels not loadable */
   SMLA_EINVAL_SCALE = -7,     /* sm_scale is not a positive finite number */
+  SMLA_EWORKSPACE_STATE = -8, /* smla_workspace_status: a launch flagged the workspace (see SMLA_WS_STATUS_*) */
   SMLA_EHIP_BASE = -100       /* HIP runtime error e is reported as SMLA_EHIP_BASE - e */
 };
 
@@ -41,7 +43,16 @@ enum {
 #define SMLA_D_V 512
 #define SMLA_FP8_RECORD_BYTES 656 /* 512 e4m3fn | 4 f32 block scales | 64 bf16 rope */
 #define SMLA_MAX_SPLITS 32
-#define SMLA_WS_COUNTER_BYTES 262144 /* head of the workspace: arrival counters, zero between calls */
+#define SMLA_WS_COUNTER_BYTES 262144 /* head of the workspace: arrival words (zero between calls) + header */
+/* The last 64 bytes of that head are the workspace header, four uint32 words written by
+ * smla_workspace_init: [0] SMLA_WS_MAGIC, [1] status (SMLA_WS_STATUS_* bits, 0 = healthy),
+ * [2] poll limit of the split merge's bounded wait, [3] reserved. */
+#define SMLA_WS_HEADER_OFFSET (SMLA_WS_COUNTER_BYTES - 64)
+#define SMLA_WS_MAGIC 0x414c4d53u          /* "SMLA" */
+#define SMLA_WS_SPIN_LIMIT_DEFAULT 4000000u /* polls (each about a microsecond) before the split merge gives up */
+#define SMLA_WS_STATUS_UNINITIALISED 1u    /* a launch found no magic word: smla_workspace_init was never run */
+#define SMLA_WS_STATUS_STALE 2u            /* an arrival word was in an illegal state (overlapping launches?) */
+#define SMLA_WS_STATUS_TIMEOUT 4u          /* the last split to arrive gave up waiting for the others */
 
 /* KV row formats */
 #define SMLA_KV_BF16 0         /* row = 576 bf16 (1152 B) */
@@ -98,7 +109,7 @@ int smla_fwd(int kv_format, const void* q, const void* kv, const int32_t* indice
 /*
  * Dense MLA decode over the whole paged context (no index list): token t of sequence s attends to
  * logical positions 0 .. seq_lens[s]-1 (clipped to max_seq_len); everything else as smla_fwd,
- * same kernels, same split merge.  seq_lens device int32 [n_tokens / tokens_per_seq], 16-byte aligned.
+ * same kernels, same split merge.  seq_lens device int32 [n_tokens / tokens_per_seq].
  * The reference's decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len,
  * attn_logits, num_kv_splits, sm_scale, page_size)
  * (/root/reference/third_party/mthreads/python/test/wmma/test_accuracy_musa_vllm_mla.py:571-620;
@@ -127,9 +138,26 @@ int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t t
 /* Bytes of workspace smla_fwd needs for the given split count (0 when n_splits <= 1). */
 size_t smla_workspace_bytes(int32_t n_tokens, int32_t n_heads, int32_t d_v, int32_t n_splits);
 
-/* Zero the arrival counters at the head of a freshly allocated workspace (a fill kernel on
- * `stream`, so it may be captured in a graph).  Needed once per allocation, not per call. */
+/* Zero the arrival words at the head of a freshly allocated workspace and write its header (a
+ * fill kernel on `stream`, so it may be captured in a graph).  Needed once per allocation, not
+ * per call. */
 int smla_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Health of a workspace after the launches issued so far.  A split launch that finds the
+ * workspace without its magic word, an arrival word in an illegal state, or whose last split
+ * waits longer than the header's poll limit for the others does not hang and does not merge: it
+ * sets a SMLA_WS_STATUS_* bit in the header, writes NaN to the LSE of the rows concerned and
+ * ends normally; until the host has dealt with it, later launches on that workspace may be
+ * flagged too.  This call waits for `stream`, copies the header back, stores the status bits in
+ * *status_out (may be NULL) and returns SMLA_OK when they were zero; otherwise it initialises
+ * the workspace again (as smla_workspace_init does, unless the magic word was missing) and
+ * returns SMLA_EWORKSPACE_STATE.  It synchronises, so it is for tests, set-up code and error
+ * handling, not for the serving loop.
+ * No counterpart in the reference (its two-stage decode keeps no state between launches:
+ * test_accuracy_musa_vllm_mla.py:426-477 is a second launch).
+ */
+int smla_workspace_status(void* workspace, size_t workspace_bytes, void* stream, uint32_t* status_out);
 
 /*
  * Page translation + masking + gather alone (the first stage of smla_fwd, exposed so the

@@ -1,8 +1,9 @@
 """CPU check of what the compiled gfx950 kernels occupy (hipcc cross-compiles without a GPU):
 every kernel's LDS fits the CU's 160 KB, and only the one kernel known to spill uses scratch.
-A spill in any other kernel is a performance regression, and spill code around loads issued
-from inline assembly is a correctness hazard (the compiler takes an asm output as written when
-the statement ends, while the load is still in flight)."""
+A spill in any other kernel is a performance regression.  Loads issued from inline assembly into
+registers are banned outright: the compiler takes an asm output as written when the statement
+ends, while the load is still in flight, so any copy or spill it places before the wait reads
+registers the hardware has not filled yet."""
 import os
 import re
 import subprocess
@@ -55,3 +56,34 @@ def test_one_wavefront_per_simd_kernels_use_the_whole_register_file():
     gemm = _resource_usage("gemm_rs.hip")
     big = [u for n, u in gemm.items() if "gemm_rs_big_kernel" in n]
     assert len(big) == 1 and big[0]["VGPRs"] + big[0]["AGPRs"] <= 128 and big[0]["LDS Size"] == 128 * 1024, big
+
+
+_LOAD_MNEMONIC = re.compile(r"\b(global_load|buffer_load|flat_load|scratch_load|ds_read|ds_load|s_load|s_buffer_load)")
+
+
+def _asm_statements(text):
+    """(line number, statement text) of every inline-assembly statement in a source file."""
+    out = []
+    for m in re.finditer(r"\basm\b\s*(?:volatile)?\s*\(", text):
+        depth, i = 1, m.end()
+        while depth and i < len(text):
+            depth += {"(": 1, ")": -1}.get(text[i], 0)
+            i += 1
+        out.append((text.count("\n", 0, m.start()) + 1, text[m.start():i]))
+    return out
+
+
+@pytest.mark.parametrize("source", sorted(f for f in os.listdir(build.CSRC) if f.endswith((".hip", ".h"))))
+def test_no_inline_asm_load_lands_in_a_register(source):
+    """Loads from inline assembly may only be direct-to-LDS moves (no register output); everything
+    that lands in a register is a load the compiler can see and count.  Every asm statement that
+    writes M0 says so in its clobber list."""
+    text = open(os.path.join(build.CSRC, source)).read()
+    for line, stmt in _asm_statements(text):
+        body = stmt.split(":")[0]
+        if _LOAD_MNEMONIC.search(body):
+            assert "_lds_" in body or " lds" in body, (source, line, "load into registers from inline asm")
+            outputs = stmt.split(":")[1] if stmt.count(":") >= 1 else ""
+            assert '"=' not in outputs and '"+' not in outputs, (source, line, "asm load with a register output")
+        if re.search(r"\bm0\b", body):
+            assert '"m0"' in stmt, (source, line, "asm writes m0 without clobbering it")
