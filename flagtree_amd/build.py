@@ -13,6 +13,8 @@ FLAGS = [
     # keep hipcc from forming packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # <smla_hw.h>: hardware-specific wrappers, found through the include path
+    "-I", CSRC,
 ]
 
 

@@ -41,8 +41,7 @@ __device__ __forceinline__ uint32_t g_pack_bf16(float a, float b) {
 }
 
 __device__ __forceinline__ g_bf16x4 g_read_tr(const uint8_t* p) {
-  g_short4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) g_short4*)(p));
-  return __builtin_bit_cast(g_bf16x4, v);
+  return hw::lds_read_tr16_b64(p);
 }
 
 __global__ __launch_bounds__(256, 2) void gemm_rs_kernel(const uint16_t* __restrict__ x,
@@ -184,6 +183,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rs_kernel(const uint16_t* __restr
 #pragma unroll
         for (int j = 0; j < 4; ++j) stage[row * kStageFloats + 32 * j + c32] = acc[i][j][r];
       }
+      hw::wave_lds_order();
 #pragma unroll
       for (int p1 = 0; p1 < 8; ++p1) {
         const int row = 2 * p1 + g;                     // within the 16 staged rows
@@ -197,6 +197,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rs_kernel(const uint16_t* __restr
         pk.y = g_pack_bf16(v.z + zz[2], v.w + zz[3]);
         *reinterpret_cast<uint2*>(o) = pk;
       }
+      hw::wave_lds_order();
     }
   }
 }
@@ -228,11 +229,10 @@ constexpr int kStage2Floats = 64;             // epilogue staging row of a wavef
 static_assert(16 * 32 * kStage2Floats * 4 <= 2 * kStage2, "epilogue staging (32 rows x 64 fp32 per wavefront) lives in the K-step buffers");
 
 __device__ __forceinline__ g_bf16x8 g_lds_b128(uint32_t a) {
-  return *(const __attribute__((address_space(3))) g_bf16x8*)(a);
+  return hw::lds_read_b128(a);
 }
 __device__ __forceinline__ g_bf16x4 g_lds_tr(uint32_t a) {
-  g_short4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) g_short4*)(a));
-  return __builtin_bit_cast(g_bf16x4, v);
+  return hw::lds_read_tr16_b64(a);
 }
 
 __global__ __launch_bounds__(1024)
@@ -262,7 +262,7 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
   }
   if (tile_m >= mt || tile_n >= nt) return;
   const int m0 = tile_m * kBM2, n0 = tile_n * kBN2;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)&s_buf[0][0];
+  const uint32_t lds0 = hw::lds_addr(&s_buf[0][0]);
 
   // ---- DMA of one K-step: 32 instructions for the X tile (8 rows each) and 32 for the W tile (2
   // rows each), 8 + 8 per wavefront.  Instruction i = 8 wave + t; the swizzles depend on i's parity
@@ -289,12 +289,12 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
       const int i = 2 * wave + d;
       const uint64_t sa = (uint64_t)(uintptr_t)x + ((uint64_t)(m0 + 8 * i) * K + k0) * 2;
       const uint32_t ma = dst + i * 1024;
-      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(a_off[d & 1]), "s"(sa), "s"(ma) : "memory", "m0");
+      hw::dma_b128(a_off[d & 1], sa, ma);
     } else {
       const int i = 2 * wave + d - 2;
       const uint64_t sb = (uint64_t)(uintptr_t)w + (uint64_t)(k0 + 2 * i) * N * 2;
       const uint32_t mb = dst + kA2Bytes + i * 1024;
-      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(b_off[d & 1]), "s"(sb), "s"(mb) : "memory", "m0");
+      hw::dma_b128(b_off[d & 1], sb, mb);
     }
   };
 
@@ -327,7 +327,7 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
     }
   };
   for (int kt = 0; kt < n_k; ++kt) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // this wavefront's share of step kt has landed
+    hw::wait_vmcnt<0>();    // this wavefront's share of step kt has landed
     __syncthreads();                                    // ... everyone's has, and everyone is done with step kt - 1
     const uint32_t buf = lds0 + (kt & 1) * kStage2;
     const bool more = kt + 1 < n_k;
@@ -395,11 +395,11 @@ int launch_gemm_rs(const void* x, const void* w, const float* partial, void* out
   const long long blocks = (long long)((mt + 7) / 8 * 8) * nt;
   if (blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
   if (big)
-    gemm_rs_big_kernel<<<dim3((unsigned)blocks), dim3(1024), 0, s>>>(
+    hipLaunchKernelGGL(gemm_rs_big_kernel, dim3((unsigned)blocks), dim3(1024), 0, s, 
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), partial, static_cast<uint16_t*>(out), m, n, k,
         m / n_chunks, (long long)chunk_stride);
   else
-    gemm_rs_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(
+    hipLaunchKernelGGL(gemm_rs_kernel, dim3((unsigned)blocks), dim3(256), 0, s, 
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), partial, static_cast<uint16_t*>(out), m, n, k,
         m / n_chunks, (long long)chunk_stride);
   return hip_status(hipGetLastError());

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <smla_hw.h>
 #include "../../include/flagtree_smla.h"
 
 namespace smla {
@@ -91,8 +92,6 @@ __device__ __forceinline__ void translate_entries4(const Params& p, int seq, int
 constexpr uint32_t kWsMagic = SMLA_WS_MAGIC;
 enum { kRolePublish = 0, kRoleLast = 1, kRoleError = 2 };
 
-typedef __attribute__((ext_vector_type(4))) uint32_t ws_u32x4;
-
 __device__ __forceinline__ void ws_flag(const Params& p, uint32_t bits) {
   __hip_atomic_fetch_or(p.ws_header + 1, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -135,16 +134,11 @@ __device__ __forceinline__ bool ws_wait_published(const Params& p, unsigned long
   return false;
 }
 
-// Partials cross workgroups without fences: stored and loaded at agent scope (sc1: through the
-// L2, past the per-CU cache), a bit is published only after the stores have been acknowledged.
-// The loads are buffer loads the compiler can see: it counts them in flight and waits where a
-// landing register is first read, whatever copies or spills it puts in between.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t ws_partial_rsrc(const float* base) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, 0x7fffffff, 0x00020000);
-}
-__device__ __forceinline__ ws_u32x4 ws_load_partial(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
-  return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 16 /* sc1 */);
-}
+// Partials cross workgroups without fences: stored and loaded at agent scope (through the L2,
+// past the per-CU cache; hw::store_b128_agent / hw::load_b128_agent), a bit is published only
+// after the stores have been acknowledged.  The loads are ones the compiler can see: it counts
+// them in flight and waits where a landing register is first read, whatever copies or spills
+// it puts in between.
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
   return __uint_as_float((uint32_t)b << 16);

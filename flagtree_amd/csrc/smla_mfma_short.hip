@@ -25,11 +25,11 @@
 namespace smla {
 namespace {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+using hw::bf16x8;
+using hw::bf16x4;
+using hw::short4v;
+using hw::f32x4;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(4))) short short4v;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 
 constexpr int kNT = 256;
@@ -52,10 +52,7 @@ template <> struct Geometry<SMLA_KV_FP8_B128> {
   static constexpr int kStageBytes = 2 * 4 * 16 * kRowLds;        // 149504: a 16-row bf16 area per wavefront (the end-of-kernel parking needs 132 KB anyway)
 };
 
-__device__ __forceinline__ bf16x4 lds_read_tr(const uint8_t* p) {
-  short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v*)(p));
-  return __builtin_bit_cast(bf16x4, v);
-}
+__device__ __forceinline__ bf16x4 lds_read_tr(const uint8_t* p) { return hw::lds_read_tr16_b64(p); }
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   bf16x2 v;
   v[0] = (__bf16)a;
@@ -85,7 +82,7 @@ __device__ __forceinline__ void dma_tile_bf16(const uint8_t* kv, const int32_t* 
     const uint8_t* src = kv + (size_t)r[i] * kRowBytesBf16 + col * 16;
     const uint32_t m0v = __builtin_amdgcn_readfirstlane(tile_lds + (4 * i + wave) * 1024);
     if (4 * i + 3 < kLoads || 4 * i + wave < kLoads) {           // wave-uniform
-      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(m0v) : "memory", "m0");
+      hw::dma_b128(src, m0v);
     }
   }
 }
@@ -225,7 +222,7 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
   for (int i = 0; i < kDvTiles; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;     // this wavefront's base-2 reference / partial row sum (lane = head)
   const float sc2 = p.sm_scale * kLog2e;
-  const uint32_t lds_ring = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)&s_ring[0];
+  const uint32_t lds_ring = hw::lds_addr(&s_ring[0]);
   constexpr int kTileRaw = kTN * G::kRawRow;
 
   int pass = kPassFast;
@@ -362,7 +359,7 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
         // bf16: the workgroup gathers 64-row tiles straight into a double-buffered LDS ring
         dma_tile_bf16(kv, s_rows, 0, n_valid, lds_ring, wave, lane);
         for (int it = 0; it < n_tiles; ++it) {
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          hw::wait_vmcnt<0>();
           __syncthreads();                   // tile `it` landed; the other ring slot is no longer read
           if (it + 1 < n_tiles)
             dma_tile_bf16(kv, s_rows, (it + 1) * kTN, n_valid, lds_ring + ((it + 1) & 1) * kTileRaw, wave, lane);
@@ -384,12 +381,16 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
         fp8_issue(kv, s_rows, kTN + 16 * wave, n_valid, lane, lb);
         for (int it = 0; it < n_my; it += 2) {
           fp8_stage(la, stage, scales, lane);
+          hw::wave_lds_order();              // the staged rows are read by other lanes of this wavefront
           fp8_issue(kv, s_rows, (it + 2) * kTN + 16 * wave, n_valid, lane, la);
           tile_math(stage, scales, min(16, n_valid - it * kTN - 16 * wave));
           if (it + 1 >= n_my) break;
+          hw::wave_lds_order();              // ... and are overwritten only after all of them have read
           fp8_stage(lb, stage, scales, lane);
+          hw::wave_lds_order();
           fp8_issue(kv, s_rows, (it + 3) * kTN + 16 * wave, n_valid, lane, lb);
           tile_math(stage, scales, min(16, n_valid - (it + 1) * kTN - 16 * wave));
+          hw::wave_lds_order();
         }
       }
     }
@@ -486,10 +487,10 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
       for (int j = 0; j < 8; ++j) {
         const float4 v = summed(j);
         const f32x4 vv = {v.x, v.y, v.z, v.w};
-        asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(o + 64 * j), "v"(vv) : "memory");
+        hw::store_b128_agent(o + 64 * j, vv);
       }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    hw::wait_vmcnt<0>();
     __syncthreads();
     if (tid == 0) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
@@ -521,7 +522,9 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
 #pragma unroll 1
   for (int i = 0; i < ns; ++i) {
     const float wi = __fmul_rn(__expf(split_lse(i) - m_ref), rw);
+    hw::wave_lds_order();
     if (q4 == 0) s_f[wave][l16] = wi;        // read back by this wavefront only (its LDS accesses complete in order)
+    hw::wave_lds_order();
     f32x4 v[8];
     if (i == sp) {
 #pragma unroll
@@ -530,10 +533,10 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
         v[j] = f32x4{a4.x, a4.y, a4.z, a4.w};
       }
     } else {
-      const __amdgpu_buffer_rsrc_t src = ws_partial_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0) * kDv);
+      const hw::buffer_rsrc src = hw::make_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0) * kDv);
       const uint32_t off = (uint32_t)((min(orow, p.n_heads - 1 - head0) * kDv + ocol) * 4);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = __builtin_bit_cast(f32x4, ws_load_partial(src, off + 256 * j));
+      for (int j = 0; j < 8; ++j) v[j] = hw::load_b128_agent(src, off + 256 * j);
     }
     const float rb = s_f[wave][orow];
 #pragma unroll
@@ -554,7 +557,7 @@ int launch_short_impl(const Params& p, hipStream_t s) {
   const int n_hblocks = (p.n_heads + 15) / 16;
   const long long blocks = ((long long)p.n_tokens + 7) / 8 * 8 * n_hblocks * p.n_splits;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
-  fwd_short_kernel<FMT><<<dim3((unsigned)blocks), dim3(kNT), 0, s>>>(p, n_hblocks);
+  hipLaunchKernelGGL(fwd_short_kernel<FMT>, dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
   return hip_status(hipGetLastError());
 }
 

@@ -28,14 +28,14 @@
 
 namespace smla {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+using hw::bf16x8;
+using hw::bf16x4;
+using hw::short4v;
+using hw::f32x4;
+using hw::u32x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(4))) short short4v;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 constexpr int kNT = 256;                      // threads per workgroup
 constexpr int kTN = 32;                       // tokens per tile
@@ -62,14 +62,8 @@ constexpr int kAccTiles = kDvHalf / 32;       // 8 accumulator tiles of 32 heads
 constexpr int kBtLdsMax = 8192;               // page-table entries that fit the staging area (32 KB of a ring slot)
 constexpr int kDmaSteps = 9;                  // DMA instructions per wavefront per tile (8 rows + 1 RoPE block)
 
-// LDS accesses by 32-bit LDS address (swizzled addresses are built with integer xor)
-__device__ __forceinline__ bf16x4 lds_read_tr(uint32_t a) {
-  short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v*)(a));
-  return __builtin_bit_cast(bf16x4, v);
-}
-__device__ __forceinline__ bf16x8 lds_read_b128(uint32_t a) {
-  return *(const __attribute__((address_space(3))) bf16x8*)(a);
-}
+using hw::lds_read_b128;
+__device__ __forceinline__ bf16x4 lds_read_tr(uint32_t a) { return hw::lds_read_tr16_b64(a); }
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   bf16x2 v;
@@ -105,7 +99,7 @@ struct DmaTile {
       const uint64_t sbase = (uint64_t)(uintptr_t)kv + (uint64_t)srow * kRowBytesBf16;
       const uint32_t m0v = tile_lds + r * kMainStride;
       const uint32_t vsw = voff ^ (uint32_t)(swz(r) << 4);
-      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(vsw), "s"(sbase), "s"(m0v) : "memory", "m0");
+      hw::dma_b128(vsw, sbase, m0v);
     } else {
       // lane l fills slot l of the 1 KB block of pairs 4*wave .. 4*wave+3
       const int pair = 4 * wave + (lane >> 4);
@@ -113,7 +107,7 @@ struct DmaTile {
       const int32_t trow = __shfl(rid, r);
       const uint8_t* src = kv + (size_t)trow * kRowBytesBf16 + 1024 + c * 16;
       const uint32_t m0v = tile_lds + kRopeBase + wave * 1024;
-      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(m0v) : "memory", "m0");
+      hw::dma_b128(src, m0v);
     }
   }
 };
@@ -293,11 +287,10 @@ __device__ __forceinline__ void tile_accumulate(uint32_t tile, uint32_t pbuf, in
 
 // s_waitcnt vmcnt(n) for a run-time n in {0, kDmaSteps, 2 * kDmaSteps}
 __device__ __forceinline__ void wait_dma(int younger_tiles) {
-  if (younger_tiles >= 2) asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
-  else if (younger_tiles == 1) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (younger_tiles >= 2) hw::wait_vmcnt<2 * kDmaSteps>();
+  else if (younger_tiles == 1) hw::wait_vmcnt<kDmaSteps>();
+  else hw::wait_vmcnt<0>();
 }
-static_assert(kDmaSteps == 9, "wait_dma encodes kDmaSteps");
 
 template <int FMT>
 __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) {
@@ -357,13 +350,13 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   const int32_t* bt_row = p.block_table ? p.block_table + (size_t)seq * p.bt_stride : nullptr;
   const bool bt_in_lds = bt_row != nullptr && p.bt_stride <= kBtLdsMax && (p.bt_stride & 3) == 0 &&
                          ((uintptr_t)bt_row & 15) == 0;
-  const uint32_t lds_bt = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)&s_tile[kSlots - 1][0];
+  const uint32_t lds_bt = hw::lds_addr(&s_tile[kSlots - 1][0]);
   if (bt_in_lds) {
     for (int c = wave; 256 * c < p.bt_stride; c += 4) {            // 1 KB (256 entries) per instruction
       const int e = 256 * c + 4 * lane;
       const uint32_t m0v = lds_bt + 1024 * c;
       if (e < p.bt_stride)
-        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(bt_row + e), "s"(m0v) : "memory", "m0");
+        hw::dma_b128(bt_row + e, m0v);
     }
   }
 
@@ -394,7 +387,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   if (bt_in_lds) {
     // Touching the index values makes the compiler wait for exactly those loads (the Q loads
     // issued behind them stay in flight); the page-table DMA is older, so it is complete as well.
-    asm volatile("" ::"v"(rr_first[0]), "v"(rr_first[1]), "v"(rr_first[2]), "v"(rr_first[3]));
+    hw::wait_for_loads_of(rr_first[0], rr_first[1], rr_first[2], rr_first[3]);
     __syncthreads();
     const int32_t* bt_s = reinterpret_cast<const int32_t*>(&s_tile[kSlots - 1][0]);
 #pragma unroll
@@ -412,8 +405,8 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // wavefronts) and this lane's partial sum over its tokens
   float m_ref[2] = {-INFINITY, -INFINITY}, l_part[2] = {0.f, 0.f};
   const float sc2 = p.sm_scale * kLog2e;
-  const uint32_t lds_tile = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)&s_tile[0][0];
-  const uint32_t lds_p = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)&s_p[0][0][0];
+  const uint32_t lds_tile = hw::lds_addr(&s_tile[0][0]);
+  const uint32_t lds_p = hw::lds_addr(&s_p[0][0][0]);
   const int partner = wave ^ 1;
 
   int pass = kPassFast;
@@ -514,13 +507,13 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
           for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ht][r], sc2, -m_ref[ht]));
           l_part[ht] += (pr[0] + pr[1]) + (pr[2] + pr[3]);
           const u32x2 w = {pack_bf16(pr[0], pr[1]), pack_bf16(pr[2], pr[3])};
-          *(__attribute__((address_space(3))) u32x2*)(pw + 16 * ht * kPStride) = w;
+          hw::lds_write_b64(pw + 16 * ht * kPStride, w);
         }
       };
 
       // ---- prologue: tiles 0 and 1 go out at once, tile 2 rides on the scores of tile 0
       if constexpr (FMT == SMLA_KV_BF16) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // Q and index loads: the DMA is counted from zero
+        hw::wait_vmcnt<0>();   // Q and index loads: the DMA is counted from zero
         for (int it = 0; it < min(n_tiles, 2); ++it) fetch_whole(it);
         wait_dma(n_tiles > 1 ? 1 : 0);
       } else {
@@ -557,8 +550,8 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
           if (it + kSlots < n_tiles) {
             const int e = min((it + kSlots) * kTN + (tid >> 3), n_valid - 1);
             const uint8_t* line = kv + (size_t)s_rows[e] * kRowBytesFp8 + min((tid & 7) * 128, kRowBytesFp8 - 4);
-            const uint32_t sink = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)&s_sink[0];
-            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(line), "s"(sink) : "memory", "m0");
+            const uint32_t sink = hw::lds_addr(&s_sink[0]);
+            hw::dma_b32(line, sink);
           }
         }
         // Tile it+1 is never the last one here, so it is full: no masking, and the reference is
@@ -582,23 +575,23 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
             const float lm = fmaxf(fmaxf(sv[i][0], sv[i][1]), fmaxf(sv[i][2], sv[i][3])) * sc2;
             m_ref[i] = pass == kPassMax ? fmaxf(m_ref[i], lm) : m_ref[i];
             over |= lm > m_ref[i] + kSlack;
-            asm volatile("" : "+v"(m_ref[i]));                     // keeps the slice where it is written
+            hw::pin(m_ref[i]);                     // keeps the slice where it is written
           } else if (i < 10) {               // slices 2..9: one probability each
             const int ht = (i - 2) >> 2, r = (i - 2) & 3;
             pr[ht][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[ht][r], sc2, -m_ref[ht]));
-            asm volatile("" : "+v"(pr[ht][r]));
+            hw::pin(pr[ht][r]);
           } else if (i < 12) {               // slices 10, 11: row sums and bf16 packing
             const int ht = i - 10;
             l_part[ht] += (pr[ht][0] + pr[ht][1]) + (pr[ht][2] + pr[ht][3]);
             pw2[ht] = u32x2{pack_bf16(pr[ht][0], pr[ht][1]), pack_bf16(pr[ht][2], pr[ht][3])};
-            asm volatile("" : "+v"(l_part[ht]), "+v"(pw2[ht]));
+            hw::pin(l_part[ht], pw2[ht]);
           } else if (i == 12) {
             failed |= pass == kPassFast && __any(over);
           }
         });
         const uint32_t pw = lds_p + (((it + 1) & 1) * 2 + hg) * kPBytes + l16 * kPStride + (16 * dh + 4 * q4) * 2;
-        *(__attribute__((address_space(3))) u32x2*)(pw) = pw2[0];
-        *(__attribute__((address_space(3))) u32x2*)(pw + 16 * kPStride) = pw2[1];
+        hw::lds_write_b64(pw, pw2[0]);
+        hw::lds_write_b64(pw + 16 * kPStride, pw2[1]);
       }
       // ---- tail: the last tiles, nothing left to fetch
       for (; it < n_tiles; ++it) {
@@ -668,6 +661,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   }
   __syncthreads();                                                 // staged blocks and scalar exchange are done
   if (g == 0) s_x[wave][c32] = inv;                                // per-row normaliser
+  hw::wave_lds_order();
   const int n_rows = min(32, p.n_heads - head0);                   // head rows that exist (wave-uniform)
   const int col4 = kDvHalf * dh + 4 * lane;                        // this lane's 4 dv columns
   auto staged = [&](int row) { return *reinterpret_cast<const float4*>(stage + row * kStageStride + 4 * lane); };
@@ -715,9 +709,9 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
       const float sc = s_x[wave][row];
       const float4 v = staged(row);
       const f32x4 vv = {__fmul_rn(v.x, sc), __fmul_rn(v.y, sc), __fmul_rn(v.z, sc), __fmul_rn(v.w, sc)};
-      asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(o + (size_t)row * kDv), "v"(vv) : "memory");
+      hw::store_b128_agent(o + (size_t)row * kDv, vv);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    hw::wait_vmcnt<0>();
     __syncthreads();
     if (tid == 0) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
@@ -760,7 +754,9 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
 #pragma unroll 1
     for (int i = 0; i < ns; ++i) {
       const float wi = __fmul_rn(__expf(split_lse(i) - m_safe), rw);
+      hw::wave_lds_order();
       if (g == 0) s_w[c32] = wi;
+      hw::wave_lds_order();
       f32x4 v[16];
       if (i == sp) {
 #pragma unroll
@@ -769,10 +765,10 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
           v[j] = f32x4{a4.x, a4.y, a4.z, a4.w};
         }
       } else {
-        const __amdgpu_buffer_rsrc_t src = ws_partial_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0) * kDv);
+        const hw::buffer_rsrc src = hw::make_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0) * kDv);
 #pragma unroll
         for (int j = 0; j < 16; ++j)
-          v[j] = __builtin_bit_cast(f32x4, ws_load_partial(src, (uint32_t)((min(r0 + j, n_rows - 1) * kDv + col4) * 4)));
+          v[j] = hw::load_b128_agent(src, (uint32_t)((min(r0 + j, n_rows - 1) * kDv + col4) * 4));
       }
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
@@ -794,7 +790,7 @@ static int launch_tall_impl(const Params& p, hipStream_t s) {
   const int n_hblocks = (p.n_heads + 63) / 64;
   const long long blocks = ((long long)p.n_tokens + 7) / 8 * 8 * n_hblocks * p.n_splits;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
-  fwd_tall_kernel<FMT><<<dim3((unsigned)blocks), dim3(kNT), 0, s>>>(p, n_hblocks);
+  hipLaunchKernelGGL(fwd_tall_kernel<FMT>, dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
   return hip_status(hipGetLastError());
 }
 

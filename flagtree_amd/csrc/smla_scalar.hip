@@ -134,9 +134,9 @@ __global__ __launch_bounds__(kScalarThreads) void fwd_scalar_kernel(Params p) {
 int launch_fwd_scalar(int kv_format, const Params& p, hipStream_t s) {
   dim3 grid(p.n_heads, p.n_tokens), block(kScalarThreads);
   switch (kv_format) {
-    case SMLA_KV_BF16: fwd_scalar_kernel<SMLA_KV_BF16, false><<<grid, block, 0, s>>>(p); break;
-    case SMLA_KV_FP8_B128: fwd_scalar_kernel<SMLA_KV_FP8_B128, false><<<grid, block, 0, s>>>(p); break;
-    case SMLA_KV_F32: fwd_scalar_kernel<SMLA_KV_F32, true><<<grid, block, 0, s>>>(p); break;
+    case SMLA_KV_BF16: hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_scalar_kernel<SMLA_KV_BF16, false>), grid, block, 0, s, p); break;
+    case SMLA_KV_FP8_B128: hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_scalar_kernel<SMLA_KV_FP8_B128, false>), grid, block, 0, s, p); break;
+    case SMLA_KV_F32: hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_scalar_kernel<SMLA_KV_F32, true>), grid, block, 0, s, p); break;
     default: return SMLA_EINVAL_SHAPE;
   }
   return hip_status(hipGetLastError());
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void gather_kernel(Params p, int row_bytes, in
 
 int launch_gather(const Params& p, int row_bytes, int32_t* phys_out, void* rows_out, hipStream_t s) {
   dim3 grid((p.topk + 3) / 4, p.n_tokens), block(256);
-  gather_kernel<<<grid, block, 0, s>>>(p, row_bytes, phys_out, static_cast<uint8_t*>(rows_out));
+  hipLaunchKernelGGL(gather_kernel, grid, block, 0, s, p, row_bytes, phys_out, static_cast<uint8_t*>(rows_out));
   return hip_status(hipGetLastError());
 }
 
@@ -201,7 +201,7 @@ int launch_merge(const float* part_out, const float* part_lse, void* out, float*
                  int n_heads, int d_v, int n_splits, hipStream_t s) {
   if (d_v != kDv) return SMLA_EINVAL_SHAPE;
   dim3 grid(n_heads, n_tokens), block(128);
-  merge_kernel<<<grid, block, 0, s>>>(part_out, part_lse, static_cast<uint16_t*>(out), lse, n_heads,
+  hipLaunchKernelGGL(merge_kernel, grid, block, 0, s, part_out, part_lse, static_cast<uint16_t*>(out), lse, n_heads,
                                       n_splits);
   return hip_status(hipGetLastError());
 }
@@ -306,7 +306,7 @@ int launch_quantize(const void* src, const int64_t* slot, void* records, int64_t
                     int64_t record_rows, hipStream_t s) {
   if (n_rows == 0) return SMLA_OK;
   dim3 grid((unsigned)((n_rows + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave))), block(256);
-  quantize_kernel<<<grid, block, 0, s>>>(static_cast<const uint16_t*>(src), slot,
+  hipLaunchKernelGGL(quantize_kernel, grid, block, 0, s, static_cast<const uint16_t*>(src), slot,
                                          static_cast<uint8_t*>(records), n_rows, record_rows);
   return hip_status(hipGetLastError());
 }
@@ -339,7 +339,7 @@ __global__ __launch_bounds__(256) void kv_copy_kernel(const uint4* __restrict__ 
 int launch_kv_copy(const void* src, const int64_t* slot, void* pool, int64_t n_rows, int64_t pool_rows, hipStream_t s) {
   if (n_rows == 0) return SMLA_OK;
   dim3 grid((unsigned)((n_rows + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave))), block(256);
-  kv_copy_kernel<<<grid, block, 0, s>>>(static_cast<const uint4*>(src), slot, static_cast<uint4*>(pool), n_rows, pool_rows);
+  hipLaunchKernelGGL(kv_copy_kernel, grid, block, 0, s, static_cast<const uint4*>(src), slot, static_cast<uint4*>(pool), n_rows, pool_rows);
   return hip_status(hipGetLastError());
 }
 
@@ -354,7 +354,7 @@ int launch_zero(void* ptr, size_t bytes, hipStream_t s) {
   const size_t n16 = bytes / 16;
   if (n16 == 0) return SMLA_OK;
   const unsigned blocks = (unsigned)((n16 + 255) / 256 > 1024 ? 1024 : (n16 + 255) / 256);
-  zero_kernel<<<dim3(blocks), dim3(256), 0, s>>>(static_cast<uint4*>(ptr), n16);
+  hipLaunchKernelGGL(zero_kernel, dim3(blocks), dim3(256), 0, s, static_cast<uint4*>(ptr), n16);
   return hip_status(hipGetLastError());
 }
 
@@ -366,7 +366,7 @@ __global__ __launch_bounds__(256) void workspace_init_kernel(uint4* __restrict__
 }
 
 int launch_workspace_init(void* workspace, hipStream_t s) {
-  workspace_init_kernel<<<dim3(64), dim3(256), 0, s>>>(static_cast<uint4*>(workspace));
+  hipLaunchKernelGGL(workspace_init_kernel, dim3(64), dim3(256), 0, s, static_cast<uint4*>(workspace));
   return hip_status(hipGetLastError());
 }
 

@@ -386,8 +386,8 @@ __global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* 
         // mask = 2 mask + (compare): a compare into vcc and an add with carry-in, two vector
         // instructions a bit (the compiler's own lowering takes three and a half); the wait state
         // between a vcc write and its use as carry-in is spelled out
-        asm("v_cmp_gt_u32 vcc, %1, %2\n\ts_nop 1\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc" : "+v"(a) : "v"(key[r][j]), "v"(thr) : "vcc");
-        asm("v_cmp_eq_u32 vcc, %1, %2\n\ts_nop 1\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc" : "+v"(e) : "v"(key[r][j]), "v"(thr) : "vcc");
+        hw::shift_in_gt_u32(a, key[r][j], thr);
+        hw::shift_in_eq_u32(e, key[r][j], thr);
       }
     }
     above[r] = a; equal[r] = e;
@@ -588,15 +588,15 @@ int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_
   // latency counts: 16 wavefronts.
   const bool many = n_rows >= 1024;
   if (n_cols <= 4096)
-    topk_resident_kernel<4, 1><<<grid, dim3(256), 0, s>>>(scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<4, 1>), grid, dim3(256), 0, s, scores, context_lens, out, n_cols, row_stride, k);
   else if (n_cols <= 16384 && many)
-    topk_resident_kernel<4, 4><<<grid, dim3(256), 0, s>>>(scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<4, 4>), grid, dim3(256), 0, s, scores, context_lens, out, n_cols, row_stride, k);
   else if (n_cols <= 16384)
-    topk_resident_kernel<16, 1><<<grid, dim3(1024), 0, s>>>(scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<16, 1>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k);
   else if (n_cols <= 65536)
-    topk_resident_kernel<16, 4><<<grid, dim3(1024), 0, s>>>(scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<16, 4>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k);
   else
-    topk_stream_kernel<16><<<grid, dim3(1024), 0, s>>>(scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_stream_kernel<16>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k);
   return hip_status(hipGetLastError());
 }
 

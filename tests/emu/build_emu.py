@@ -1,0 +1,60 @@
+"""Build the kernel sources for the CPU emulator (test infrastructure; the product never loads it).
+
+The very same .hip files the product compiles for gfx950 are compiled here as host C++ against
+tests/emu/include (a stand-in <hip/hip_runtime.h> and <smla_hw.h>), together with the fiber
+runtime, into tests/emu/libflagtree_smla_emu.so.  ``python tests/emu/build_emu.py``."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+CSRC = os.path.join(ROOT, "flagtree_amd", "csrc")
+LIB_PATH = os.path.join(HERE, "libflagtree_smla_emu.so")
+SOURCES = ["smla_api.hip", "smla_scalar.hip", "smla_mfma_tall.hip", "smla_mfma_short.hip", "gemm_rs.hip", "topk_select.hip"]
+CXX = os.environ.get("EMU_CXX", "/opt/rocm/llvm/bin/clang++")
+FLAGS = ["-x", "c++", "-std=c++17", "-O2", "-g1", "-fPIC", "-ffp-contract=off", "-fno-strict-aliasing",
+         "-Wno-unused-value", "-Wno-pass-failed", "-Wno-unknown-attributes", "-Wno-ignored-attributes",
+         "-I", os.path.join(HERE, "include"), "-I", CSRC]
+
+
+def _stale(outputs, inputs):
+    if not all(os.path.exists(o) for o in outputs):
+        return True
+    newest = max(os.path.getmtime(i) for i in inputs)
+    return any(os.path.getmtime(o) < newest for o in outputs)
+
+
+def build(verbose=False, force=False):
+    headers = [os.path.join(HERE, "emu_runtime.h"), os.path.join(HERE, "include", "smla_hw.h"),
+               os.path.join(HERE, "include", "hip", "hip_runtime.h"), os.path.join(CSRC, "smla_common.h"),
+               os.path.join(ROOT, "include", "flagtree_smla.h"), os.path.abspath(__file__)]
+    objs = []
+    procs = []
+    for src in SOURCES + ["emu_runtime.cc"]:
+        path = os.path.join(HERE if src.endswith(".cc") else CSRC, src)
+        obj = os.path.join(HERE, "build", src + ".o")
+        objs.append(obj)
+        if not force and not _stale([obj], [path] + headers):
+            continue
+        os.makedirs(os.path.dirname(obj), exist_ok=True)
+        cmd = [CXX] + FLAGS + ["-c", path, "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for src, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError(f"emulator build of {src} failed:\n{out[-6000:]}")
+        if verbose and out.strip():
+            print(out)
+    if procs or not os.path.exists(LIB_PATH):
+        res = subprocess.run([CXX, "-shared", "-o", LIB_PATH] + objs, stdout=subprocess.PIPE,
+                             stderr=subprocess.STDOUT, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("emulator link failed:\n" + res.stdout[-4000:])
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose="-q" not in sys.argv, force="-f" in sys.argv))

@@ -1,0 +1,301 @@
+// Fiber scheduler, rendezvous, LDS arena and deferred global -> LDS moves of the CPU emulator.
+#include "emu_runtime.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <sys/mman.h>
+
+#include <algorithm>
+#include <random>
+#include <vector>
+
+extern "C" char __start_emu_lds[];
+extern "C" char __stop_emu_lds[];
+
+// void emu_switch(void** save_sp, void* load_sp): x86-64 SysV context switch (callee-saved registers + stack)
+asm(R"(
+.text
+.globl emu_switch
+.type emu_switch,@function
+emu_switch:
+  pushq %rbp
+  pushq %rbx
+  pushq %r12
+  pushq %r13
+  pushq %r14
+  pushq %r15
+  movq %rsp, (%rdi)
+  movq %rsi, %rsp
+  popq %r15
+  popq %r14
+  popq %r13
+  popq %r12
+  popq %rbx
+  popq %rbp
+  ret
+.size emu_switch,.-emu_switch
+)");
+extern "C" void emu_switch(void** save_sp, void* load_sp);
+
+namespace emu {
+
+namespace {
+
+constexpr size_t kStackBytes = 256 * 1024;
+
+struct Fiber {
+  Lane lane;
+  void* sp = nullptr;
+  char* stack = nullptr;
+  bool done = false;
+  // what the fiber is waiting for: runnable once *wait_gen differs from wait_val (null: runnable)
+  const unsigned long long* wait_gen = nullptr;
+  unsigned long long wait_val = 0;
+  struct Pending { uint32_t lds_dst; int bytes; uint8_t data[16]; };
+  std::vector<Pending> dma;
+};
+
+}  // namespace
+
+struct Wave {
+  int n_lanes = 0;                 // lanes that exist
+  int live = 0;                    // lanes that have not left the kernel
+  int arrived = 0;
+  unsigned long long gen = 0;      // completed rendezvous
+  uint32_t tag = 0;
+  bool lane_live[kWave];
+  alignas(64) uint8_t slot[2][kWave][kSlotBytes];
+};
+
+namespace {
+
+struct Block {
+  std::vector<Fiber> fibers;
+  std::vector<Wave> waves;
+  int live = 0;
+  int arrived = 0;
+  unsigned long long gen = 0;
+};
+
+Block g_block;
+Fiber* g_cur = nullptr;
+void* g_sched_sp = nullptr;
+Dim3 g_block_idx, g_block_dim, g_grid_dim;
+const std::function<void()>* g_body = nullptr;
+int g_dma_eager = 0;
+unsigned g_order_seed = 0;
+unsigned long long g_launches = 0;
+std::vector<char*> g_stacks;
+
+void yield() { emu_switch(&g_cur->sp, g_sched_sp); }
+
+void leave_wave(Fiber* f) {
+  Wave* w = f->lane.wave;
+  w->lane_live[f->lane.lane] = false;
+  w->live--;
+  // a rendezvous the others are waiting in may now be complete
+  if (w->live > 0 && w->arrived == w->live) { w->arrived = 0; w->gen++; }
+  g_block.live--;
+  if (g_block.live > 0 && g_block.arrived == g_block.live) { g_block.arrived = 0; g_block.gen++; }
+}
+
+void fiber_main() {
+  Fiber* f = g_cur;
+  (*g_body)();
+  f->dma.clear();
+  f->done = true;
+  leave_wave(f);
+  yield();
+  fail("a finished fiber was resumed");
+}
+
+char* get_stack(size_t i) {
+  while (g_stacks.size() <= i) {
+    void* p = mmap(nullptr, kStackBytes, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    if (p == MAP_FAILED) fail("mmap of a fiber stack failed");
+    g_stacks.push_back(static_cast<char*>(p));
+  }
+  return g_stacks[i];
+}
+
+void prepare(Fiber* f) {
+  uintptr_t top = (reinterpret_cast<uintptr_t>(f->stack) + kStackBytes) & ~uintptr_t(15);
+  void** s = reinterpret_cast<void**>(top);
+  *--s = nullptr;                                   // return address of fiber_main (never used)
+  *--s = reinterpret_cast<void*>(&fiber_main);      // `ret` of the first switch lands here
+  for (int i = 0; i < 6; ++i) *--s = nullptr;       // rbp rbx r12 r13 r14 r15
+  f->sp = s;
+}
+
+void run_block(Dim3 bidx) {
+  const unsigned n = g_block_dim.x * g_block_dim.y * g_block_dim.z;
+  const unsigned n_waves = (n + kWave - 1) / kWave;
+  g_block_idx = bidx;
+  g_block.fibers.assign(n, Fiber());
+  g_block.waves.assign(n_waves, Wave());
+  g_block.live = (int)n;
+  g_block.arrived = 0;
+  g_block.gen = 0;
+  memset(__start_emu_lds, 0xFB, __stop_emu_lds - __start_emu_lds);   // LDS holds no defined values at workgroup start
+  for (unsigned i = 0; i < n; ++i) {
+    Fiber& f = g_block.fibers[i];
+    Wave& w = g_block.waves[i / kWave];
+    f.lane.flat = (int)i;
+    f.lane.lane = (int)(i % kWave);
+    f.lane.tid = Dim3(i % g_block_dim.x, (i / g_block_dim.x) % g_block_dim.y, i / (g_block_dim.x * g_block_dim.y));
+    f.lane.wave = &w;
+    w.n_lanes++;
+    w.live++;
+    w.lane_live[i % kWave] = true;
+    f.stack = get_stack(i);
+    prepare(&f);
+  }
+  for (Wave& w : g_block.waves)
+    for (int l = w.n_lanes; l < kWave; ++l) w.lane_live[l] = false;
+  // round-robin until every lane has left; a full round without any lane finishing or any
+  // rendezvous completing means the lanes are waiting for each other in different places
+  unsigned long long idle_rounds = 0;
+  while (g_block.live > 0) {
+    unsigned long long before = g_block.gen;
+    for (Wave& w : g_block.waves) before += w.gen;
+    const int live_before = g_block.live;
+    for (Fiber& f : g_block.fibers) {
+      if (f.done) continue;
+      if (f.wait_gen != nullptr && *f.wait_gen == f.wait_val) continue;
+      f.wait_gen = nullptr;
+      g_cur = &f;
+      emu_switch(&g_sched_sp, f.sp);
+    }
+    unsigned long long after = g_block.gen;
+    for (Wave& w : g_block.waves) after += w.gen;
+    if (after == before && g_block.live == live_before) {
+      if (++idle_rounds > 4)
+        fail("deadlock in block (%u,%u,%u): %d lanes wait at barriers that cannot complete", bidx.x, bidx.y, bidx.z, g_block.live);
+    } else {
+      idle_rounds = 0;
+    }
+  }
+  g_cur = nullptr;
+}
+
+}  // namespace
+
+void fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  fprintf(stderr, "[emu] ");
+  vfprintf(stderr, fmt, ap);
+  fprintf(stderr, "\n");
+  va_end(ap);
+  fflush(stderr);
+  abort();
+}
+
+Lane* self() { return &g_cur->lane; }
+Dim3 block_idx() { return g_block_idx; }
+Dim3 block_dim() { return g_block_dim; }
+Dim3 grid_dim() { return g_grid_dim; }
+
+int wave_rendezvous(const void* post, size_t bytes, uint32_t tag) {
+  Fiber* f = g_cur;
+  Wave* w = f->lane.wave;
+  if (bytes > (size_t)kSlotBytes) fail("rendezvous operand of %zu bytes", bytes);
+  const unsigned long long my_gen = w->gen;
+  const int parity = (int)(my_gen & 1);
+  if (bytes) memcpy(w->slot[parity][f->lane.lane], post, bytes);
+  if (w->arrived == 0) w->tag = tag;
+  else if (w->tag != tag)
+    fail("block (%u,%u,%u) wave %d: lanes reached different wave-wide operations (tags %08x / %08x): "
+         "a collective inside divergent control flow", g_block_idx.x, g_block_idx.y, g_block_idx.z,
+         f->lane.flat / kWave, w->tag, tag);
+  w->arrived++;
+  if (w->arrived == w->live) {
+    w->arrived = 0;
+    w->gen++;
+  } else {
+    f->wait_gen = &w->gen;
+    f->wait_val = my_gen;
+    yield();
+  }
+  return parity;
+}
+
+const uint8_t* wave_slot(int parity, int lane) { return g_cur->lane.wave->slot[parity][lane]; }
+bool wave_lane_live(int lane) { return g_cur->lane.wave->lane_live[lane]; }
+
+void block_barrier() {
+  const unsigned long long my_gen = g_block.gen;
+  g_block.arrived++;
+  if (g_block.arrived == g_block.live) {
+    g_block.arrived = 0;
+    g_block.gen++;
+  } else {
+    g_cur->wait_gen = &g_block.gen;
+    g_cur->wait_val = my_gen;
+    yield();
+  }
+}
+
+uint32_t lds_addr(const void* p) {
+  const char* c = static_cast<const char*>(p);
+  if (c < __start_emu_lds || c > __stop_emu_lds) fail("lds_addr of an object outside LDS");
+  return (uint32_t)(c - __start_emu_lds);
+}
+
+uint8_t* lds_ptr(uint32_t addr, size_t bytes) {
+  const size_t size = (size_t)(__stop_emu_lds - __start_emu_lds);
+  if ((size_t)addr + bytes > size)
+    fail("LDS access out of bounds: address %u + %zu, arena %zu (block (%u,%u,%u), thread %d)", addr, bytes, size,
+         g_block_idx.x, g_block_idx.y, g_block_idx.z, g_cur ? g_cur->lane.flat : -1);
+  return reinterpret_cast<uint8_t*>(__start_emu_lds) + addr;
+}
+
+void dma_issue(const void* src, uint32_t lds_dst, int bytes) {
+  if (bytes != 4 && bytes != 16) fail("dma of %d bytes per lane", bytes);
+  if (g_dma_eager) {
+    memcpy(lds_ptr(lds_dst, bytes), src, bytes);
+    return;
+  }
+  Fiber::Pending p;
+  p.lds_dst = lds_dst;
+  p.bytes = bytes;
+  memcpy(p.data, src, bytes);
+  lds_ptr(lds_dst, bytes);                           // bounds check at issue
+  g_cur->dma.push_back(p);
+}
+
+void dma_wait(int allowed_in_flight) {
+  std::vector<Fiber::Pending>& q = g_cur->dma;
+  const size_t keep = std::min(q.size(), (size_t)std::max(allowed_in_flight, 0));
+  const size_t land = q.size() - keep;
+  for (size_t i = 0; i < land; ++i) memcpy(lds_ptr(q[i].lds_dst, q[i].bytes), q[i].data, q[i].bytes);
+  q.erase(q.begin(), q.begin() + land);
+}
+
+void launch(Dim3 grid, Dim3 block, const std::function<void()>& body) {
+  if (g_cur != nullptr) fail("launch from inside a kernel");
+  g_launches++;
+  g_block_dim = block;
+  g_grid_dim = grid;
+  g_body = &body;
+  const size_t n_blocks = (size_t)grid.x * grid.y * grid.z;
+  std::vector<size_t> order(n_blocks);
+  for (size_t i = 0; i < n_blocks; ++i) order[i] = i;
+  if (g_order_seed) {
+    std::mt19937 rng(g_order_seed);
+    std::shuffle(order.begin(), order.end(), rng);
+  }
+  for (size_t i : order)
+    run_block(Dim3((unsigned)(i % grid.x), (unsigned)((i / grid.x) % grid.y), (unsigned)(i / ((size_t)grid.x * grid.y))));
+  g_body = nullptr;
+}
+
+}  // namespace emu
+
+extern "C" {
+void emu_set_dma_mode(int eager) { emu::g_dma_eager = eager; }
+void emu_set_block_order(unsigned seed) { emu::g_order_seed = seed; }
+unsigned long long emu_launch_count(void) { return emu::g_launches; }
+}

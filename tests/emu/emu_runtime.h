@@ -1,0 +1,69 @@
+// CPU emulator for the kernels' execution model: test infrastructure only, never part of the
+// product.  One OS thread runs a workgroup's lanes as cooperative fibers; operations that involve
+// a whole wavefront (cross-lane moves, ballots, matrix instructions, transposing LDS reads) and
+// workgroup barriers are rendezvous points.  Workgroups of a launch run one after another.
+//
+// What it models beyond plain arithmetic:
+//   * wave64 lane semantics of every cross-lane operation the kernels use,
+//   * register layouts of the MFMA instructions and of ds_read_b64_tr_b16,
+//   * LDS as one arena addressed by 32-bit addresses, trashed before every workgroup,
+//   * global -> LDS moves that complete late (at the wait) or early (at issue), selectable,
+//     so that both a missing wait and a slot overwritten too soon change the results,
+//   * a collective reached by only part of a wavefront's live lanes aborts with a message.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#include <functional>
+
+namespace emu {
+
+struct Dim3 {
+  unsigned x, y, z;
+  constexpr Dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
+};
+
+constexpr int kWave = 64;
+constexpr int kSlotBytes = 128;        // operand bytes a lane can post per collective
+
+struct Wave;
+struct Lane {
+  Dim3 tid;
+  int lane;                            // lane id in its wavefront
+  int flat;                            // thread id in the workgroup
+  Wave* wave;
+};
+
+Lane* self();                          // the lane that is running now
+Dim3 block_idx();
+Dim3 block_dim();
+Dim3 grid_dim();
+
+// Rendezvous of the live lanes of the calling lane's wavefront.  `tag` names the operation; lanes
+// arriving with different tags (divergent control flow around a collective) abort the process.
+// Returns the parity of the slot set posted for this rendezvous.
+int wave_rendezvous(const void* post, size_t bytes, uint32_t tag);
+const uint8_t* wave_slot(int parity, int lane);      // what `lane` posted (valid until the next rendezvous but one)
+bool wave_lane_live(int lane);                       // lane exists and has not left the kernel
+void block_barrier();
+
+// LDS arena: every __shared__ object lives in the ELF section "emu_lds"
+uint32_t lds_addr(const void* p);
+uint8_t* lds_ptr(uint32_t addr, size_t bytes);       // bounds-checked
+
+// global -> LDS moves
+void dma_issue(const void* src, uint32_t lds_dst, int bytes);
+void dma_wait(int allowed_in_flight);
+
+void launch(Dim3 grid, Dim3 block, const std::function<void()>& body);
+
+[[noreturn]] void fail(const char* fmt, ...);
+
+}  // namespace emu
+
+extern "C" {
+// knobs for the tests
+void emu_set_dma_mode(int eager);        // 0: moves land at the wait (default), 1: at issue
+void emu_set_block_order(unsigned seed); // 0: ascending block ids, else a seeded shuffle
+unsigned long long emu_launch_count(void);
+}

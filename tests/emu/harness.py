@@ -1,0 +1,102 @@
+"""Calls into the emulator build of the kernel sources (tests only).
+
+The emulated library exports the same C ABI as the product library; here it is given CPU tensors,
+whose memory the emulated kernels read and write directly."""
+import ctypes
+import importlib.util
+import math
+import os
+
+import torch
+
+from flagtree_amd import _lib as product_lib
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        spec = importlib.util.spec_from_file_location("build_emu", os.path.join(HERE, "build_emu.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        path = mod.build()
+        l = ctypes.CDLL(path)
+        for name, (res, args) in product_lib.SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        l.emu_set_dma_mode.argtypes = [ctypes.c_int]
+        l.emu_set_block_order.argtypes = [ctypes.c_uint]
+        l.emu_launch_count.restype = ctypes.c_ulonglong
+        _lib = l
+    return _lib
+
+
+def configure(dma_eager=False, block_order_seed=0):
+    l = lib()
+    l.emu_set_dma_mode(1 if dma_eager else 0)
+    l.emu_set_block_order(block_order_seed)
+
+
+_FORMATS = {"bf16": 0, "fp8_e4m3_b128": 1, "f32": 2}
+
+
+def make_workspace(n_bytes):
+    ws = torch.empty(max(int(n_bytes), product_lib.SMLA_WS_COUNTER_BYTES), dtype=torch.uint8)
+    ws.fill_(0xA5)
+    rc = lib().smla_workspace_init(ws.data_ptr(), ws.numel(), None)
+    assert rc == 0, rc
+    return ws
+
+
+def workspace_status(ws):
+    status = ctypes.c_uint32(0)
+    rc = lib().smla_workspace_status(ws.data_ptr(), ws.numel(), None, ctypes.byref(status))
+    return rc, status.value
+
+
+def forward(cfg, n_splits=1, workspace=None, dense_lens=None, scalar=False):
+    """cfg as flagtree_amd.workloads builds it, on the CPU.  Returns (out [T, H, 512], lse [T, H], rc)."""
+    l = lib()
+    q = cfg["q"]
+    H, D = q.shape[-2], q.shape[-1]
+    q3 = q.reshape(-1, H, D).contiguous()
+    T = q3.shape[0]
+    bt = cfg.get("block_table")
+    B = q.shape[0] if q.dim() == 4 else (bt.shape[0] if bt is not None else 1)
+    S = T // B
+    kvc = cfg["kv_cache"]
+    kv2 = kvc.reshape(-1, kvc.shape[-1]).contiguous()
+    stride = 0
+    if bt is None and kvc.dim() >= 3 and kvc.shape[0] == B and B > 1:
+        stride = kvc[0].numel() // kvc.shape[-1]
+    fmt = _FORMATS[cfg["kv_format"]]
+    out = torch.full((T, H, 512), float("nan"), dtype=q.dtype)
+    lse = torch.full((T, H), float("nan"), dtype=torch.float32)
+    btc = bt.contiguous() if bt is not None else None
+    bt_ptr = btc.data_ptr() if btc is not None else None
+    bt_stride = btc.shape[1] if btc is not None else 0
+    sm = float(cfg.get("sm_scale", 1.0 / math.sqrt(576)))
+    if scalar:
+        idx = cfg["indices"].reshape(T, -1).to(torch.int32).contiguous()
+        rc = l.smla_fwd_scalar(fmt, q3.data_ptr(), kv2.data_ptr(), idx.data_ptr(), bt_ptr, out.data_ptr(), lse.data_ptr(),
+                               T, S, H, idx.shape[1], 576, 512, cfg["page_size"], bt_stride, stride, kv2.shape[0], sm, None)
+        return out, lse, rc
+    ws_bytes = l.smla_workspace_bytes(T, H, 512, n_splits)
+    if ws_bytes and workspace is None:
+        workspace = make_workspace(ws_bytes)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_n = workspace.numel() if workspace is not None else 0
+    if dense_lens is not None:
+        lens = dense_lens.to(torch.int32).contiguous()
+        rc = l.smla_decode_dense(fmt, q3.data_ptr(), kv2.data_ptr(), lens.data_ptr(), bt_ptr, out.data_ptr(), lse.data_ptr(),
+                                 T, S, H, bt_stride * cfg["page_size"], 576, 512, cfg["page_size"], bt_stride, stride,
+                                 kv2.shape[0], sm, n_splits, ws_ptr, ws_n, None)
+    else:
+        idx = cfg["indices"].reshape(T, -1).to(torch.int32).contiguous()
+        rc = l.smla_fwd(fmt, q3.data_ptr(), kv2.data_ptr(), idx.data_ptr(), bt_ptr, out.data_ptr(), lse.data_ptr(),
+                        T, S, H, idx.shape[1], 576, 512, cfg["page_size"], bt_stride, stride, kv2.shape[0], sm,
+                        n_splits, ws_ptr, ws_n, None)
+    return out, lse, rc

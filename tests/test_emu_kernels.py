@@ -1,0 +1,306 @@
+"""The kernel sources themselves, run on the CPU emulator (tests/emu) against the oracle.
+
+No GPU is involved: the very .hip files the product compiles for gfx950 are compiled as host
+code against a stand-in HIP header and executed lane by lane (fibers), with the cross-lane
+operations, matrix-instruction layouts, LDS addressing and global -> LDS moves modelled.  What
+this checks is the kernels' logic -- indexing, swizzles, masking, pipelining and waits, split
+merge, edge cases -- to the same bars as the GPU parity tests (bit-exact for integer and byte
+work; out max-abs <= 1e-2, lse <= 1e-3).  It says nothing about speed, and instruction-level
+hazards (registers, spills, cache coherence) are outside its model.
+
+Every forward case runs twice: with the global -> LDS moves landing as late as the kernel allows
+(at its waits) and as early as possible (at issue); a missing wait fails the first, a ring slot
+refilled too soon the second.  Split launches also run with the workgroups in a shuffled order,
+so that every split gets to be the one that merges."""
+import ctypes
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from _util import max_abs, oracle_inputs, run_oracle, to_np
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "emu"))
+import harness  # noqa: E402
+
+OUT_TOL = 1e-2
+LSE_TOL = 1e-3
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _emulator():
+    harness.lib()
+    yield
+    harness.configure()
+
+
+def _check(cfg, out, lse, out_tol=OUT_TOL, lse_tol=LSE_TOL):
+    ro, rl = run_oracle(cfg)
+    H = cfg["q"].shape[-2]
+    eo = max_abs(to_np(out).reshape(-1, H, 512), ro)
+    el = max_abs(to_np(lse).reshape(-1, H), rl)
+    assert eo <= out_tol, f"out max-abs {eo}"
+    assert el <= lse_tol, f"lse max-abs {el}"
+
+
+def _forward_all_ways(cfg, n_splits, **kw):
+    """Forward under every emulator setting; results must agree bit for bit.  Returns (out, lse)."""
+    results = []
+    settings = [(False, 0), (True, 0)] + ([(False, 12345), (True, 777)] if n_splits > 1 else [])
+    for eager, order in settings:
+        harness.configure(dma_eager=eager, block_order_seed=order)
+        out, lse, rc = harness.forward(cfg, n_splits=n_splits, **kw)
+        assert rc == 0, rc
+        results.append((out, lse))
+    harness.configure()
+    for out, lse in results[1:]:
+        assert torch.equal(out.view(torch.int16) if out.dtype == torch.bfloat16 else out,
+                           results[0][0].view(torch.int16) if out.dtype == torch.bfloat16 else results[0][0])
+        assert torch.equal(lse, results[0][1])
+    return results[0]
+
+
+def _fp8_cfg(batch, heads, pages_per_seq, topk, seed=1004, pad_frac=0.0):
+    """decode_fp8 recipe on the CPU: records written by the emulated cache writer."""
+    from flagtree_amd import workloads
+    g = torch.Generator().manual_seed(seed)
+    n_pages = batch * pages_per_seq
+    rows = n_pages * 64
+    bt = torch.randperm(n_pages, generator=g).to(torch.int32).view(batch, pages_per_seq)
+    latent = (torch.randn((rows, 576), generator=g) * 0.1).to(torch.bfloat16)
+    rec = torch.zeros((rows, 656), dtype=torch.uint8)
+    rc = harness.lib().smla_kv_quantize_fp8(latent.data_ptr(), None, rec.data_ptr(), rows, rows, None)
+    assert rc == 0
+    q = (torch.randn((batch, 1, heads, 576), generator=g) * 0.1).to(torch.bfloat16)
+    idx = workloads._topk_indices(batch, pages_per_seq * 64, topk, int(pad_frac * topk), g, True)
+    return dict(q=q, kv_cache=rec.view(n_pages, 64, 656), indices=idx.view(batch, 1, topk), block_table=bt,
+                page_size=64, sm_scale=workloads.SM_SCALE, kv_format="fp8_e4m3_b128", name="decode_fp8"), latent
+
+
+# ---- forward kernels --------------------------------------------------------------------------
+
+@pytest.mark.parametrize("heads,n_splits", [(128, 1), (128, 2), (64, 3), (96, 1), (40, 2)])
+def test_many_heads_kernel_bf16(heads, n_splits):
+    from flagtree_amd import workloads
+    cfg = workloads.decode_bf16("cpu", batch=2, heads=heads, pages_per_seq=10, topk=390, pad_frac=0.07)
+    out, lse = _forward_all_ways(cfg, n_splits)
+    _check(cfg, out, lse)
+
+
+@pytest.mark.parametrize("heads,n_splits", [(16, 1), (16, 2), (8, 1), (32, 2), (24, 1)])
+def test_few_heads_kernel_bf16(heads, n_splits):
+    from flagtree_amd import workloads
+    cfg = workloads.decode_bf16("cpu", batch=2, heads=heads, pages_per_seq=10, topk=330, pad_frac=0.07)
+    out, lse = _forward_all_ways(cfg, n_splits)
+    _check(cfg, out, lse)
+
+
+@pytest.mark.parametrize("heads,n_splits", [(16, 1), (16, 2), (128, 1), (128, 2), (8, 1)])
+def test_fp8_records(heads, n_splits):
+    cfg, _ = _fp8_cfg(2, heads, 6, 300, pad_frac=0.03)
+    out, lse = _forward_all_ways(cfg, n_splits)
+    _check(cfg, out, lse)
+
+
+def test_more_than_one_chunk_of_the_list():
+    """Lists longer than the 1024 entries the kernels compact at a time, ragged last tile."""
+    from flagtree_amd import workloads
+    for heads in (128, 16):
+        cfg = workloads.decode_bf16("cpu", batch=1, heads=heads, pages_per_seq=40, topk=2100, pad_frac=0.05)
+        out, lse = _forward_all_ways(cfg, 1)
+        _check(cfg, out, lse)
+
+
+def test_plumbing_f32_scalar_kernel():
+    from flagtree_amd import workloads
+    cfg = workloads.plumbing_f32("cpu", tokens=2, heads=16, s_kv=512, topk=64)
+    out, lse, rc = harness.forward(cfg, n_splits=1)
+    assert rc == 0
+    _check(cfg, out, lse, out_tol=2e-6, lse_tol=2e-5)
+    cfg = workloads.decode_bf16("cpu", batch=2, heads=16, pages_per_seq=8, topk=100, pad_frac=0.1)
+    out, lse, rc = harness.forward(cfg, scalar=True)
+    assert rc == 0
+    _check(cfg, out, lse, out_tol=2e-3, lse_tol=1e-5)
+
+
+def test_causal_prefill_reduced():
+    from flagtree_amd import workloads
+    cfg = workloads.prefill_causal_bf16("cpu", tokens=40, heads=128, topk=48)
+    out, lse = _forward_all_ways(cfg, 1)
+    idx = to_np(cfg["indices"]).reshape(40, 48)
+    assert (idx[0] >= 0).sum() == 1 and (idx[39] >= 0).sum() == 40
+    _check(cfg, out, lse)
+
+
+@pytest.mark.parametrize("heads", [128, 16])
+def test_edge_cases(heads):
+    g = torch.Generator().manual_seed(7)
+    kv = (torch.randn((300, 576), generator=g) * 0.1).to(torch.bfloat16)
+    q = (torch.randn((6, heads, 576), generator=g) * 0.1).to(torch.bfloat16)
+    idx = torch.full((6, 70), -1, dtype=torch.int32)
+    idx[1, 33] = 5                                           # single valid entry
+    idx[2, :] = torch.randperm(300, generator=g)[:70].to(torch.int32)   # all valid, ragged top-k (70)
+    idx[3, :35] = 17                                         # duplicates count once per occurrence
+    idx[4, ::2] = torch.arange(35, dtype=torch.int32)        # interleaved padding
+    idx[5, 0] = 299
+    idx[5, 1] = 300                                          # out of range -> masked
+    cfg = dict(q=q, kv_cache=kv, indices=idx, block_table=None, page_size=64, sm_scale=576 ** -0.5, kv_format="bf16")
+    for ns in (1, 2):
+        out, lse = _forward_all_ways(cfg, ns)
+        _check(cfg, out, lse)
+        o, l = to_np(out), to_np(lse)
+        assert (o[0] == 0).all() and np.isneginf(l[0]).all()          # token without valid entries
+        assert np.array_equal(o[1], np.broadcast_to(to_np(kv)[5, :512], (heads, 512)))   # K = 1: out = v
+
+
+@pytest.mark.parametrize("heads", [128, 16])
+def test_wide_score_range_takes_the_redo_passes(heads):
+    """Scores that outgrow the first tile's maximum by more than the slack force the exact
+    two-pass path; outputs reach 4, so the bar is relative."""
+    g = torch.Generator().manual_seed(11)
+    kv = (torch.randn((400, 576), generator=g) * 4.0).to(torch.bfloat16)
+    kv[:64] *= 0.01                                          # a first tile with tiny scores
+    q = (torch.randn((2, heads, 576), generator=g) * 4.0).to(torch.bfloat16)
+    idx = torch.arange(200, dtype=torch.int32).repeat(2, 1)
+    cfg = dict(q=q, kv_cache=kv, indices=idx, block_table=None, page_size=64, sm_scale=576 ** -0.5, kv_format="bf16")
+    ro, rl = run_oracle(cfg)
+    for ns in (1, 2):
+        out, lse = _forward_all_ways(cfg, ns)
+        assert max_abs(to_np(lse), rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
+        assert max_abs(to_np(out), ro) <= 1.2e-2 * max(1.0, float(np.abs(ro).max()))
+
+
+@pytest.mark.parametrize("heads,fmt", [(128, "bf16"), (16, "bf16"), (16, "fp8")])
+def test_dense_decode(heads, fmt):
+    from flagtree_amd import workloads
+    if fmt == "fp8":
+        cfg, _ = _fp8_cfg(3, heads, 5, 64)
+    else:
+        cfg = workloads.decode_bf16("cpu", batch=3, heads=heads, pages_per_seq=5, topk=64, pad_frac=0.0)
+    lens = torch.tensor([300, 1, 129], dtype=torch.int32)
+    out, lse = _forward_all_ways(cfg, 2, dense_lens=lens)
+    listed = dict(cfg)
+    idx = torch.full((3, 1, 320), -1, dtype=torch.int32)
+    for b, n in enumerate(lens.tolist()):
+        idx[b, 0, :n] = torch.arange(n, dtype=torch.int32)
+    listed["indices"] = idx
+    _check(listed, out, lse)
+
+
+# ---- split workspace: failure handling --------------------------------------------------------
+
+def _words(ws):
+    from flagtree_amd import _lib
+    return ws[:_lib.SMLA_WS_HEADER_OFFSET].view(torch.int64)
+
+
+def _header(ws):
+    from flagtree_amd import _lib
+    return ws[_lib.SMLA_WS_HEADER_OFFSET:_lib.SMLA_WS_HEADER_OFFSET + 16].view(torch.int32)
+
+
+@pytest.mark.parametrize("heads", [128, 16])
+@pytest.mark.parametrize("stale", ["one ticket", "own bit", "all ones"])
+def test_stale_arrival_word_is_flagged_not_hung(heads, stale):
+    from flagtree_amd import _lib, workloads
+    cfg = workloads.decode_bf16("cpu", batch=3, heads=heads, pages_per_seq=6, topk=260, pad_frac=0.05)
+    ref_out, ref_lse, rc = harness.forward(cfg, n_splits=1)
+    assert rc == 0
+    n_hblocks = (heads + 63) // 64 if heads > 32 else (heads + 15) // 16
+    ws = harness.make_workspace(harness.lib().smla_workspace_bytes(3, heads, 512, 2))
+    _header(ws)[2] = 50
+    _words(ws)[1 * n_hblocks] = {"one ticket": 1 << 32, "own bit": 1, "all ones": -1}[stale]
+    out, lse, rc = harness.forward(cfg, n_splits=2, workspace=ws)
+    assert rc == 0
+    rc, status = harness.workspace_status(ws)
+    assert rc == _lib.SMLA_EWORKSPACE_STATE and status & (2 | 4)
+    per_block = 64 if heads > 32 else 16
+    l = to_np(lse)
+    assert np.isnan(l[1, :min(per_block, heads)]).all()
+    assert max_abs(l[[0, 2]], to_np(ref_lse)[[0, 2]]) <= 1e-3
+    assert harness.workspace_status(ws) == (0, 0)
+    assert int((_words(ws) != 0).sum()) == 0
+    out2, lse2, rc = harness.forward(cfg, n_splits=2, workspace=ws)
+    assert rc == 0 and harness.workspace_status(ws) == (0, 0)
+    assert max_abs(to_np(lse2), to_np(ref_lse)) <= 1e-3 and max_abs(to_np(out2), to_np(ref_out)) <= 1e-2
+
+
+def test_uninitialised_workspace_is_flagged():
+    from flagtree_amd import _lib, workloads
+    cfg = workloads.decode_bf16("cpu", batch=2, heads=128, pages_per_seq=6, topk=260, pad_frac=0.05)
+    ws = torch.zeros(harness.lib().smla_workspace_bytes(2, 128, 512, 2), dtype=torch.uint8)
+    out, lse, rc = harness.forward(cfg, n_splits=2, workspace=ws)
+    assert rc == 0
+    rc, status = harness.workspace_status(ws)
+    assert rc == _lib.SMLA_EWORKSPACE_STATE and status & 1
+    assert np.isnan(to_np(lse)).all()
+
+
+# ---- integer / byte paths: bit-exact ------------------------------------------------------------
+
+def test_gather_and_translation_bit_exact():
+    from flagtree_amd import workloads
+    cfg = workloads.decode_bf16("cpu", batch=5, heads=16, pages_per_seq=8, topk=96, pad_frac=0.2)
+    idx = cfg["indices"].clone().view(5, 96)
+    idx[0, 0] = -1
+    idx[1, 50] = 8 * 64
+    idx[2, 95] = 2 ** 31 - 1
+    idx[3, :] = -1
+    kv = cfg["kv_cache"].view(torch.int16).reshape(-1, 576).contiguous()
+    bt = cfg["block_table"].contiguous()
+    phys = torch.full((5, 96), -7, dtype=torch.int32)
+    rows = torch.full((5, 96, 576), -7, dtype=torch.int16)
+    rc = harness.lib().smla_gather_rows(kv.data_ptr(), 1152, idx.data_ptr(), bt.data_ptr(), phys.data_ptr(), rows.data_ptr(),
+                                        5, 1, 96, 64, bt.shape[1], 0, kv.shape[0], None)
+    assert rc == 0
+    want = oracle.translate_indices(to_np(idx), to_np(bt), 64, kv_rows=kv.shape[0])
+    assert np.array_equal(to_np(phys).astype(np.int64), want)
+    assert np.array_equal(to_np(rows), oracle.gather_rows(to_np(kv), want))
+
+
+def test_cache_writer_bit_exact():
+    g = torch.Generator().manual_seed(3)
+    latent = (torch.randn((200, 576), generator=g) * torch.logspace(-3, 2, 200).view(-1, 1)).to(torch.bfloat16)
+    latent[5, 100:228] = 0                                   # an all-zero block
+    slots = torch.randperm(260, generator=g)[:200].to(torch.int64) - 20
+    for fmt, code, width, dtype in (("fp8_e4m3_b128", 1, 656, torch.uint8), ("bf16", 0, 576, torch.bfloat16)):
+        cache = torch.zeros((220, width), dtype=dtype)
+        rc = harness.lib().smla_kv_write(code, latent.data_ptr(), slots.data_ptr(), cache.data_ptr(), 200, 220, None)
+        assert rc == 0
+        want = np.zeros((220, width), dtype=np.uint8 if fmt != "bf16" else np.uint16)
+        want = oracle.reshape_and_cache(to_np(latent), want, slots.numpy(), kv_format=fmt)
+        got = cache.numpy() if fmt != "bf16" else cache.view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(got, want), fmt
+
+
+@pytest.mark.parametrize("rows,n,k", [(3, 4096, 2048), (2, 1000, 64), (1, 20000, 300), (2, 70000, 128), (5, 33, 40)])
+def test_topk_indices_exact(rows, n, k):
+    g = torch.Generator().manual_seed(rows * 131 + n)
+    scores = torch.randn((rows, n), generator=g)
+    scores[0, : n // 3] = scores[0, 0]                        # ties across the selection boundary
+    scores[-1, 5 % n] = float("nan")
+    lens = torch.randint(1, n + 1, (rows,), generator=g, dtype=torch.int32)
+    out = torch.full((rows, k), -9, dtype=torch.int32)
+    rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), rows, n, n, k, None)
+    assert rc == 0
+    assert np.array_equal(to_np(out), oracle.topk_indices(to_np(scores), k, to_np(lens)))
+
+
+@pytest.mark.parametrize("m,n,k,chunks", [(256, 256, 128, 2), (128, 512, 192, 1), (384, 256, 64, 3), (512, 256, 128, 4)])
+def test_local_gemm(m, n, k, chunks):
+    g = torch.Generator().manual_seed(m + n + k)
+    x = (torch.randn((m, k), generator=g) * 0.1).to(torch.bfloat16)
+    w = (torch.randn((k, n), generator=g) * 0.1).to(torch.bfloat16)
+    partial = torch.randn((m, n), generator=g)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16)
+    for eager in (False, True):
+        harness.configure(dma_eager=eager)
+        rc = harness.lib().smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), partial.data_ptr(), out.data_ptr(), m, n, k, chunks,
+                                              (m // chunks) * n, None)
+        assert rc == 0
+        want = oracle.gemm_rs_local(to_np(x), to_np(w), to_np(partial), n_chunks=chunks).reshape(m, n)
+        assert max_abs(to_np(out), want) <= 1e-2 + 1e-2 * float(np.abs(want).max())
+    harness.configure()
