@@ -23,7 +23,7 @@ SIGNATURES = {
     "smla_fwd": (_c.c_int, [_c.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
                             _i32, _i32, _i64, _i64, _f32, _i32, _vp, _sz, _vp]),
     "smla_decode_dense": (_c.c_int, [_c.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
-                                     _i32, _i32, _i64, _i64, _f32, _i32, _vp, _sz, _vp]),
+                                     _i32, _i32, _i64, _i64, _f32, _f32, _i32, _vp, _sz, _vp]),
     "smla_fwd_scalar": (_c.c_int, [_c.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
                                    _i32, _i32, _i32, _i64, _i64, _f32, _vp]),
     "smla_plan_splits": (_c.c_int, [_c.c_int, _i32, _i32, _i32]),

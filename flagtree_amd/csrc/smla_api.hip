@@ -49,7 +49,7 @@ const char* smla_strerror(int status) {
     case SMLA_EINVAL_WORKSPACE: return "workspace missing or too small";
     case SMLA_EINVAL_SPLITS: return "n_splits out of range for this top-k length";
     case SMLA_ENODEVICE: return "no usable gfx950 device";
-    case SMLA_EINVAL_SCALE: return "sm_scale must be positive and finite";
+    case SMLA_EINVAL_SCALE: return "sm_scale must be positive and finite, logit_cap non-negative and finite";
     case SMLA_EWORKSPACE_STATE: return "a split launch flagged its workspace (uninitialised, shared by overlapping launches, or a split never arrived)";
     default: break;
   }
@@ -57,7 +57,7 @@ const char* smla_strerror(int status) {
   return "unknown status";
 }
 
-int smla_abi_version(void) { return 1; }
+int smla_abi_version(void) { return 2; }
 
 // Workspace layout: [0, SMLA_WS_HEADER_OFFSET) arrival words (zero between calls), the 64-byte
 // header {magic, status, poll limit, -} up to SMLA_WS_COUNTER_BYTES, then the partial outputs [T, n_splits, H, d_v] f32 and the partial LSEs [T, n_splits, H] f32.
@@ -126,7 +126,7 @@ static int fill_params(Params& p, const void* q, const void* kv, const int32_t* 
   p.n_tokens = n_tokens; p.tokens_per_seq = tokens_per_seq; p.n_heads = n_heads; p.topk = topk;
   p.page_size = block_table ? page_size : 1; p.bt_stride = block_table ? bt_stride : 0;
   p.n_splits = 1; p.split_len = topk;
-  p.kv_seq_stride = kv_seq_stride; p.kv_rows = kv_rows; p.sm_scale = sm_scale;
+  p.kv_seq_stride = kv_seq_stride; p.kv_rows = kv_rows; p.sm_scale = sm_scale; p.logit_cap = 0.f;
   return SMLA_OK;
 }
 
@@ -136,7 +136,7 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
                     const int32_t* block_table, void* out, float* lse, int32_t n_tokens,
                     int32_t tokens_per_seq, int32_t n_heads, int32_t topk, int32_t d_qk, int32_t d_v,
                     int32_t page_size, int32_t block_table_stride, int64_t kv_seq_stride, int64_t kv_rows,
-                    float sm_scale, int32_t n_splits, void* workspace, size_t workspace_bytes,
+                    float sm_scale, float logit_cap, int32_t n_splits, void* workspace, size_t workspace_bytes,
                     void* stream) {
   int rc = check_common(q, kv, indices, out, lse, n_tokens, tokens_per_seq, n_heads, topk, d_qk, d_v,
                         page_size, block_table, block_table_stride, kv_seq_stride, kv_rows);
@@ -150,6 +150,8 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
   fill_params(p, q, kv, indices, block_table, out, lse, n_tokens, tokens_per_seq, n_heads, topk,
               page_size, block_table_stride, kv_seq_stride, kv_rows, sm_scale);
   if (dense) { p.seq_lens = indices; p.indices = nullptr; }
+  if (!(logit_cap >= 0.f) || !(logit_cap < INFINITY)) return SMLA_EINVAL_SCALE;
+  p.logit_cap = logit_cap;
   if (kv_format == SMLA_KV_F32) return launch_fwd_scalar(kv_format, p, s);
 
   if (n_splits == 0) {
@@ -182,7 +184,7 @@ int smla_fwd(int kv_format, const void* q, const void* kv, const int32_t* indice
              float sm_scale, int32_t n_splits, void* workspace, size_t workspace_bytes,
              void* stream) {
   return fwd_impl(false, kv_format, q, kv, indices, block_table, out, lse, n_tokens, tokens_per_seq, n_heads,
-                  topk, d_qk, d_v, page_size, block_table_stride, kv_seq_stride, kv_rows, sm_scale, n_splits,
+                  topk, d_qk, d_v, page_size, block_table_stride, kv_seq_stride, kv_rows, sm_scale, 0.f, n_splits,
                   workspace, workspace_bytes, stream);
 }
 
@@ -190,10 +192,10 @@ int smla_decode_dense(int kv_format, const void* q, const void* kv, const int32_
                       const int32_t* block_table, void* out, float* lse, int32_t n_tokens,
                       int32_t tokens_per_seq, int32_t n_heads, int32_t max_seq_len, int32_t d_qk,
                       int32_t d_v, int32_t page_size, int32_t block_table_stride, int64_t kv_seq_stride,
-                      int64_t kv_rows, float sm_scale, int32_t n_splits, void* workspace,
+                      int64_t kv_rows, float sm_scale, float logit_cap, int32_t n_splits, void* workspace,
                       size_t workspace_bytes, void* stream) {
   return fwd_impl(true, kv_format, q, kv, seq_lens, block_table, out, lse, n_tokens, tokens_per_seq, n_heads,
-                  max_seq_len, d_qk, d_v, page_size, block_table_stride, kv_seq_stride, kv_rows, sm_scale,
+                  max_seq_len, d_qk, d_v, page_size, block_table_stride, kv_seq_stride, kv_rows, sm_scale, logit_cap,
                   n_splits, workspace, workspace_bytes, stream);
 }
 

@@ -33,6 +33,22 @@ struct Params {
   int32_t page_size, bt_stride, n_splits, split_len;
   int64_t kv_seq_stride, kv_rows;
   float sm_scale;
+  float logit_cap;              // > 0: every scaled score s becomes logit_cap * tanh(s / logit_cap) before the softmax
+};
+
+// The capped score in the base-2 units the softmax works in:
+//   log2(e) * cap * tanh(x / cap),  x = raw dot product * sm_scale,
+// with tanh(y) = 1 - 2 / (exp(2 y) + 1): one exponential and one reciprocal per score.  Exact at
+// both ends (exp2 -> inf gives cap, exp2 -> 0 gives -cap); the cancellation near 0 costs an
+// absolute error of a few 1e-7 * cap, far inside the 1e-3 bar on the LSE.
+struct LogitCap {
+  float a, b;                   // a = 2 log2(e) sm_scale / cap,  b = log2(e) cap
+  __device__ __forceinline__ LogitCap(float sm_scale, float cap)
+      : a(2.f * 1.4426950408889634f * sm_scale / cap), b(1.4426950408889634f * cap) {}
+  __device__ __forceinline__ float operator()(float raw) const {
+    const float e = __builtin_amdgcn_exp2f(raw * a);
+    return __builtin_fmaf(-2.f * b, __builtin_amdgcn_rcpf(e + 1.f), b);
+  }
 };
 
 // Entry j of token t's list: the index list itself, or (dense attention over the whole context)
@@ -181,7 +197,7 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
 }
 
 int launch_fwd_scalar(int kv_format, const Params& p, hipStream_t s);
-int launch_fwd_tall(int kv_format, const Params& p, hipStream_t s);    // n_heads > 32
+int launch_fwd_tall(int kv_format, const Params& p, hipStream_t s);    // n_heads > 32 (logit cap: a second instantiation)
 int launch_fwd_short(int kv_format, const Params& p, hipStream_t s);   // n_heads <= 32
 int launch_merge(const float* part_out, const float* part_lse, void* out, float* lse,
                  int n_tokens, int n_heads, int d_v, int n_splits, hipStream_t s);

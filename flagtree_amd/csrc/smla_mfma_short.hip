@@ -149,7 +149,7 @@ __device__ __forceinline__ void fp8_stage(const u32x4 (&L)[kFp8Loads], uint8_t* 
 // reference and never moves it, so the accumulators are only ever touched by MFMA.
 // Probabilities may exceed 1, by at most 2^kSlack; if a later score exceeds the reference by more
 // the workgroup redoes its split in two passes (exact maxima, then the accumulation).
-template <int FMT>
+template <int FMT, bool CAP>
 __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks) {
   using G = Geometry<FMT>;
   __shared__ __attribute__((aligned(16))) uint8_t s_ring[G::kRingBytes + G::kStageBytes];   // ring, then staging
@@ -221,7 +221,10 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
 #pragma unroll
   for (int i = 0; i < kDvTiles; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;     // this wavefront's base-2 reference / partial row sum (lane = head)
-  const float sc2 = p.sm_scale * kLog2e;
+  // raw dot product -> base-2 exponent: one multiply, or (logit cap) the squashed score, which
+  // already is in base-2 units
+  const float sc2 = CAP ? 1.f : p.sm_scale * kLog2e;
+  [[maybe_unused]] const LogitCap cap(p.sm_scale, CAP ? p.logit_cap : 1.f);
   const uint32_t lds_ring = hw::lds_addr(&s_ring[0]);
   constexpr int kTileRaw = kTN * G::kRawRow;
 
@@ -299,6 +302,10 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
             s[r] = sacc[4][r] + sacc[0][r] * scl[r].x + sacc[1][r] * scl[r].y + sacc[2][r] * scl[r].z + sacc[3][r] * scl[r].w;
         } else {
           s = sacc[0] + sacc[1];
+        }
+        if constexpr (CAP) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[r] = cap(s[r]);
         }
         if (my_valid < 16) {
 #pragma unroll
@@ -552,20 +559,22 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
   if (tid == 0) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
 }
 
-template <int FMT>
+template <int FMT, bool CAP>
 int launch_short_impl(const Params& p, hipStream_t s) {
   const int n_hblocks = (p.n_heads + 15) / 16;
   const long long blocks = ((long long)p.n_tokens + 7) / 8 * 8 * n_hblocks * p.n_splits;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
-  hipLaunchKernelGGL(fwd_short_kernel<FMT>, dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_short_kernel<FMT, CAP>), dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
   return hip_status(hipGetLastError());
 }
 
 }  // namespace
 
 int launch_fwd_short(int kv_format, const Params& p, hipStream_t s) {
-  if (kv_format == SMLA_KV_BF16) return launch_short_impl<SMLA_KV_BF16>(p, s);
-  if (kv_format == SMLA_KV_FP8_B128) return launch_short_impl<SMLA_KV_FP8_B128>(p, s);
+  const bool cap = p.logit_cap > 0.f;
+  if (kv_format == SMLA_KV_BF16) return cap ? launch_short_impl<SMLA_KV_BF16, true>(p, s) : launch_short_impl<SMLA_KV_BF16, false>(p, s);
+  if (kv_format == SMLA_KV_FP8_B128)
+    return cap ? launch_short_impl<SMLA_KV_FP8_B128, true>(p, s) : launch_short_impl<SMLA_KV_FP8_B128, false>(p, s);
   return SMLA_EINVAL_SHAPE;
 }
 

@@ -292,7 +292,7 @@ __device__ __forceinline__ void wait_dma(int younger_tiles) {
   else hw::wait_vmcnt<0>();
 }
 
-template <int FMT>
+template <int FMT, bool CAP>
 __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) {
   __shared__ __attribute__((aligned(1024))) uint8_t s_tile[kSlots][kTileBytes];   // swizzle xors need 1 KB alignment
   __shared__ __attribute__((aligned(16))) uint8_t s_p[2][2][kPBytes];             // [tile parity][head group]
@@ -404,7 +404,10 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // softmax state of heads 16*ht + lane%16 (ht = 0, 1): base-2 reference (common to the pair of
   // wavefronts) and this lane's partial sum over its tokens
   float m_ref[2] = {-INFINITY, -INFINITY}, l_part[2] = {0.f, 0.f};
-  const float sc2 = p.sm_scale * kLog2e;
+  // raw dot product -> base-2 exponent: one multiply, or (logit cap) the squashed score, which
+  // already is in base-2 units
+  const float sc2 = CAP ? 1.f : p.sm_scale * kLog2e;
+  [[maybe_unused]] const LogitCap cap(p.sm_scale, CAP ? p.logit_cap : 1.f);
   const uint32_t lds_tile = hw::lds_addr(&s_tile[0][0]);
   const uint32_t lds_p = hw::lds_addr(&s_p[0][0][0]);
   const int partner = wave ^ 1;
@@ -474,6 +477,10 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
         tile_scores(tile, 16 * dh, qf, sa, lane, side);
         s[0] = sa[0] + sa[1];
         s[1] = sa[2] + sa[3];
+        if constexpr (CAP) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) { s[0][r] = cap(s[0][r]); s[1][r] = cap(s[1][r]); }
+        }
         if (my_valid < 16) {                 // ragged tile (uniform): mask the rows past the end
 #pragma unroll
           for (int r = 0; r < 4; ++r)
@@ -572,6 +579,10 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
             // (per-lane maximum only: the overflow test does not need the row maximum, and a
             // maximum pass folds the lanes of a head together when it ends)
             sv[i] = sa[2 * i] + sa[2 * i + 1];
+            if constexpr (CAP) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) sv[i][r] = cap(sv[i][r]);
+            }
             const float lm = fmaxf(fmaxf(sv[i][0], sv[i][1]), fmaxf(sv[i][2], sv[i][3])) * sc2;
             m_ref[i] = pass == kPassMax ? fmaxf(m_ref[i], lm) : m_ref[i];
             over |= lm > m_ref[i] + kSlack;
@@ -785,18 +796,20 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   if (tid == 0) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
 }
 
-template <int FMT>
+template <int FMT, bool CAP>
 static int launch_tall_impl(const Params& p, hipStream_t s) {
   const int n_hblocks = (p.n_heads + 63) / 64;
   const long long blocks = ((long long)p.n_tokens + 7) / 8 * 8 * n_hblocks * p.n_splits;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
-  hipLaunchKernelGGL(fwd_tall_kernel<FMT>, dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_tall_kernel<FMT, CAP>), dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
   return hip_status(hipGetLastError());
 }
 
 int launch_fwd_tall(int kv_format, const Params& p, hipStream_t s) {
-  if (kv_format == SMLA_KV_BF16) return launch_tall_impl<SMLA_KV_BF16>(p, s);
-  if (kv_format == SMLA_KV_FP8_B128) return launch_tall_impl<SMLA_KV_FP8_B128>(p, s);
+  const bool cap = p.logit_cap > 0.f;
+  if (kv_format == SMLA_KV_BF16) return cap ? launch_tall_impl<SMLA_KV_BF16, true>(p, s) : launch_tall_impl<SMLA_KV_BF16, false>(p, s);
+  if (kv_format == SMLA_KV_FP8_B128)
+    return cap ? launch_tall_impl<SMLA_KV_FP8_B128, true>(p, s) : launch_tall_impl<SMLA_KV_FP8_B128, false>(p, s);
   return SMLA_EINVAL_SHAPE;
 }
 

@@ -83,7 +83,11 @@ __global__ __launch_bounds__(kScalarThreads) void fwd_scalar_kernel(Params p) {
         for (int i = 0; i < kDqk / 64; ++i) part += s_q[lane + 64 * i] * R::get(row, lane + 64 * i);
       }
       part = wave_sum(part);
-      if (lane == 0) s_score[j] = r >= 0 ? part * p.sm_scale : -INFINITY;
+      if (lane == 0) {
+        float sc = part * p.sm_scale;
+        if (p.logit_cap > 0.f) sc = p.logit_cap * tanhf(sc / p.logit_cap);
+        s_score[j] = r >= 0 ? sc : -INFINITY;
+      }
     }
     __syncthreads();
     float m_loc = -INFINITY;

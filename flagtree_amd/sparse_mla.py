@@ -389,10 +389,11 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len, attn
                    ignored (there is one kernel)
       attn_logits  the reference's split scratch [B, H, splits, 513]; accepted and ignored (the
                    library's own workspace holds the split partials)
-      logit_cap    must be 0 (the tanh cap of the reference is not implemented)
+      logit_cap    > 0: every scaled score s becomes ``logit_cap * tanh(s / logit_cap)`` before the
+                   softmax (reference :299-302); 0 = off
     Returns (o, lse) with lse [B, H] fp32, natural log."""
-    if logit_cap != 0.0:
-        raise NotImplementedError("logit_cap is not supported")
+    if not (0.0 <= float(logit_cap) < float("inf")):
+        raise ValueError("logit_cap must be non-negative and finite (0 = off)")
     if q.dim() != 3 or q.shape[-1] != D_QK:
         raise ValueError("q must be [B, H, 576]")
     for name, t in (("q", q), ("k_buffer", k_buffer), ("req_to_token", req_to_token), ("b_seq_len", b_seq_len)):
@@ -439,6 +440,6 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len, attn
     kv_rows = k_buffer.numel() // row
     rc = lib.smla_decode_dense(fmt, q3.data_ptr(), k_buffer.data_ptr(), seq.data_ptr(), bt.data_ptr(), o.data_ptr(),
                                lse.data_ptr(), B, 1, H, max_len, D_QK, D_V, int(page_size), bt.shape[1], 0, kv_rows,
-                               float(sm_scale), eff, ws_ptr, ws_bytes, _stream(q))
+                               float(sm_scale), float(logit_cap), eff, ws_ptr, ws_bytes, _stream(q))
     _lib.check(rc, "smla_decode_dense")
     return o, lse

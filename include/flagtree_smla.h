@@ -34,7 +34,7 @@ enum {
   SMLA_EINVAL_WORKSPACE = -4, /* workspace missing or too small for n_splits > 1 */
   SMLA_EINVAL_SPLITS = -5,    /* n_splits outside [1, SMLA_MAX_SPLITS] */
   SMLA_ENODEVICE = -6,        /* no gfx950 device / kernels not loadable */
-  SMLA_EINVAL_SCALE = -7,     /* sm_scale is not a positive finite number */
+  SMLA_EINVAL_SCALE = -7,     /* sm_scale is not a positive finite number, or logit_cap is negative / not finite */
   SMLA_EWORKSPACE_STATE = -8, /* smla_workspace_status: a launch flagged the workspace (see SMLA_WS_STATUS_*) */
   SMLA_EHIP_BASE = -100       /* HIP runtime error e is reported as SMLA_EHIP_BASE - e */
 };
@@ -110,8 +110,10 @@ int smla_fwd(int kv_format, const void* q, const void* kv, const int32_t* indice
  * Dense MLA decode over the whole paged context (no index list): token t of sequence s attends to
  * logical positions 0 .. seq_lens[s]-1 (clipped to max_seq_len); everything else as smla_fwd,
  * same kernels, same split merge.  seq_lens device int32 [n_tokens / tokens_per_seq].
+ * logit_cap > 0 squashes every scaled score s to logit_cap * tanh(s / logit_cap) before the
+ * mask and the softmax (0 = off), as the reference's kernels do (:299-302).
  * The reference's decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len,
- * attn_logits, num_kv_splits, sm_scale, page_size)
+ * attn_logits, num_kv_splits, sm_scale, page_size, logit_cap)
  * (/root/reference/third_party/mthreads/python/test/wmma/test_accuracy_musa_vllm_mla.py:571-620;
  * page lookup :278-283) for a latent cache whose values are the first d_v columns of its keys.
  */
@@ -119,8 +121,8 @@ int smla_decode_dense(int kv_format, const void* q, const void* kv, const int32_
                       const int32_t* block_table, void* out, float* lse,
                       int32_t n_tokens, int32_t tokens_per_seq, int32_t n_heads, int32_t max_seq_len,
                       int32_t d_qk, int32_t d_v, int32_t page_size, int32_t block_table_stride,
-                      int64_t kv_seq_stride, int64_t kv_rows, float sm_scale, int32_t n_splits,
-                      void* workspace, size_t workspace_bytes, void* stream);
+                      int64_t kv_seq_stride, int64_t kv_rows, float sm_scale, float logit_cap,
+                      int32_t n_splits, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Same computation with the exact-fp32 scalar kernel regardless of shape; q/kv/out dtype
  * follows kv_format (bf16 inputs are widened to fp32, out is written in the q dtype).

@@ -75,9 +75,16 @@ def gather_rows(rows, phys):
     return out
 
 
-def sparse_mla_fwd(q, kv, phys, sm_scale, d_v=512, dtype=np.float64):
+def sparse_mla_fwd(q, kv, phys, sm_scale, d_v=512, dtype=np.float64, logit_cap=0.0):
     """q [T, H, D], kv [N, D] (already dequantised values), phys [T, K] physical
-    row ids with -1 = invalid  ->  (out [T, H, d_v], lse [T, H]) in ``dtype``."""
+    row ids with -1 = invalid  ->  (out [T, H, d_v], lse [T, H]) in ``dtype``.
+
+    ``logit_cap`` > 0 squashes every scaled score before the mask and the maximum, as the
+    reference's MLA decode kernels do: ``qk = logit_cap * tanh(qk / logit_cap)`` after
+    ``qk *= sm_scale`` (/root/reference/third_party/mthreads/python/test/wmma/
+    test_accuracy_musa_vllm_mla.py:299-302, :109-111).  Pinned by tests/test_oracle_mla.py: a
+    per-element loop with math.tanh, the equal-keys closed form lse = cap tanh(s / cap) + log n,
+    the bound lse <= cap + log n, and the limit cap -> infinity (no cap)."""
     q = np.asarray(q, dtype=dtype)
     kv = np.asarray(kv, dtype=dtype)
     phys = np.asarray(phys)
@@ -90,6 +97,8 @@ def sparse_mla_fwd(q, kv, phys, sm_scale, d_v=512, dtype=np.float64):
             continue
         rows = kv[sel]                                   # [n, D]
         s = (q[t] @ rows.T) * dtype(sm_scale)            # [H, n]
+        if logit_cap > 0:
+            s = dtype(logit_cap) * np.tanh(s / dtype(logit_cap))
         m = s.max(axis=1, keepdims=True)
         e = np.exp(s - m)
         l = e.sum(axis=1, keepdims=True)

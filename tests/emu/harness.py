@@ -57,7 +57,7 @@ def workspace_status(ws):
     return rc, status.value
 
 
-def forward(cfg, n_splits=1, workspace=None, dense_lens=None, scalar=False):
+def forward(cfg, n_splits=1, workspace=None, dense_lens=None, scalar=False, logit_cap=0.0):
     """cfg as flagtree_amd.workloads builds it, on the CPU.  Returns (out [T, H, 512], lse [T, H], rc)."""
     l = lib()
     q = cfg["q"]
@@ -93,7 +93,7 @@ def forward(cfg, n_splits=1, workspace=None, dense_lens=None, scalar=False):
         lens = dense_lens.to(torch.int32).contiguous()
         rc = l.smla_decode_dense(fmt, q3.data_ptr(), kv2.data_ptr(), lens.data_ptr(), bt_ptr, out.data_ptr(), lse.data_ptr(),
                                  T, S, H, bt_stride * cfg["page_size"], 576, 512, cfg["page_size"], bt_stride, stride,
-                                 kv2.shape[0], sm, n_splits, ws_ptr, ws_n, None)
+                                 kv2.shape[0], sm, float(logit_cap), n_splits, ws_ptr, ws_n, None)
     else:
         idx = cfg["indices"].reshape(T, -1).to(torch.int32).contiguous()
         rc = l.smla_fwd(fmt, q3.data_ptr(), kv2.data_ptr(), idx.data_ptr(), bt_ptr, out.data_ptr(), lse.data_ptr(),

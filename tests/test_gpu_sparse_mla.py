@@ -375,9 +375,44 @@ def test_decode_attention_fwd_dense(dev, H, page_size, fmt):
            "page_size": page_size, "kv_format": fmt, "sm_scale": 576 ** -0.5}
     wo, wl = run_oracle(cfg)
     assert max_abs(to_np(o), wo.reshape(B, H, 512)) <= 1e-2 and max_abs(to_np(lse), wl.reshape(B, H)) <= 1e-3
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):
         ft.decode_attention_fwd(q.to(dev), k_buffer, v_buffer, o, req_to_token.to(dev), lens.to(dev), None, None,
-                                576 ** -0.5, page_size, logit_cap=30.0)
+                                576 ** -0.5, page_size, logit_cap=-1.0)
+
+
+@pytest.mark.parametrize("H,fmt,std,cap,min_diff", [(128, "bf16", 1.5, 2.0, 0.5), (16, "bf16", 1.5, 2.0, 0.5),
+                                                    (16, "fp8_e4m3_b128", 1.5, 2.0, 0.5), (64, "fp8_e4m3_b128", 0.5, 0.2, 0.01)])
+@pytest.mark.parametrize("splits", [1, 2])
+def test_decode_attention_fwd_logit_cap(dev, H, fmt, std, cap, min_diff, splits):
+    """logit_cap * tanh(score / logit_cap) before the softmax (reference test_accuracy_musa_vllm_mla.py:299-302);
+    inputs scaled so that raw scores reach several times the cap.  (The many-heads kernel rounds
+    dequantised fp8 values to bf16 when it stages them, an error that grows with the square of the
+    input scale: its case stays nearer the benchmark's magnitudes.)"""
+    import flagtree_amd as ft
+    g = torch.Generator().manual_seed(77 + H)
+    B, L, page_size = 3, 700, 64
+    lens = torch.tensor([L, 3, 300], dtype=torch.int32)
+    n_pages = -(-L // page_size)
+    req_to_token = torch.randperm(2 * B * n_pages, generator=g)[:B * n_pages].to(torch.int32).view(B, n_pages)
+    lat = (torch.randn((2 * B * n_pages * page_size, 576), generator=g) * std).to(torch.bfloat16)
+    q = (torch.randn((B, H, 576), generator=g) * std).to(torch.bfloat16)
+    if fmt == "bf16":
+        k_buffer = lat.to(dev).view(-1, page_size, 576)
+    else:
+        k_buffer = ft.quantize_kv_fp8(lat.to(dev)).view(-1, page_size, 656)
+    o, lse = ft.decode_attention_fwd(q.to(dev), k_buffer, None, None, req_to_token.to(dev), lens.to(dev), None, splits,
+                                     576 ** -0.5, page_size, logit_cap=cap)
+    max_len = n_pages * page_size
+    idx = torch.arange(max_len, dtype=torch.int32).repeat(B, 1)
+    idx[idx >= lens[:, None]] = -1
+    cfg = {"q": q.view(B, 1, H, 576), "indices": idx.view(B, 1, max_len), "kv_cache": k_buffer, "block_table": req_to_token,
+           "page_size": page_size, "kv_format": fmt, "sm_scale": 576 ** -0.5}
+    qn, kv_small, phys_small, _ = oracle_inputs(cfg)
+    wo, wl = oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfg["sm_scale"], 512, logit_cap=cap)
+    uo, ul = oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfg["sm_scale"], 512)
+    assert max_abs(wl, ul) > min_diff                                   # the cap matters on these inputs
+    assert max_abs(to_np(lse), wl.reshape(B, H)) <= 1e-3
+    assert max_abs(to_np(o), wo.reshape(B, H, 512)) <= 1e-2 * max(1.0, float(np.abs(wo).max()))
 
 
 @pytest.mark.parametrize("heads,ns", [(128, 2), (128, 4), (16, 2), (16, 8)])

@@ -33,13 +33,13 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
         assert hasattr(lib, n), f"{n} declared in include/flagtree_smla.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.smla_abi_version() == 1
+    assert lib.smla_abi_version() == 2
 
 
 def test_status_texts(lib):
     from flagtree_amd import _lib
     assert _lib.strerror(0) == "ok"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         assert _lib.strerror(code) not in ("ok", "unknown status")
     with pytest.raises(ValueError):
         _lib.check(-2, "x")
@@ -91,10 +91,11 @@ def test_validation_codes_without_a_device(lib):
         a = dict(ok, **kw)
         return lib.smla_decode_dense(a["fmt"], a["q"], a["kv"], a["idx"], a["bt"], a["out"], a["lse"], a["T"], a["S"], a["H"],
                                      a["K"], a["dqk"], a["dv"], a["page"], a["bts"], a["stride"], a["rows"], a["scale"],
-                                     a["ns"], a["ws"], a["wsb"], a["stream"])
+                                     a.get("cap", 0.0), a["ns"], a["ws"], a["wsb"], a["stream"])
 
     assert dense(q=None) == -1 and dense(idx=None) == -1 and dense(dv=256) == -2 and dense(K=0) == -2
     assert dense(out=p16 + 2) == -3 and dense(ns=40) == -5 and dense(scale=float("nan")) == -7
+    assert dense(cap=-1.0) == -7 and dense(cap=float("inf")) == -7 and dense(cap=float("nan")) == -7
 
     def scalar(**kw):
         a = dict(ok, **kw)

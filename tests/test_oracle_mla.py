@@ -183,3 +183,43 @@ def test_topk_indices_against_repeated_maximum():
     idx = oracle.topk_indices(x, 32)
     for r in range(4):
         assert np.array_equal(np.sort(x[r, idx[r]])[::-1], np.sort(x[r])[::-1][:32])
+
+
+def test_logit_cap_closed_forms_and_loop():
+    """cap * tanh(score / cap) before the softmax (reference test_accuracy_musa_vllm_mla.py:299-302)."""
+    import math
+    rng = np.random.default_rng(5)
+    T, H, D, N, K = 2, 3, 576, 40, 17
+    q = rng.standard_normal((T, H, D)) * 2.0
+    kv = rng.standard_normal((N, D)) * 2.0
+    phys = np.stack([rng.permutation(N)[:K] for _ in range(T)])
+    phys[0, 3] = -1
+    scale, cap = 576 ** -0.5, 1.5                        # raw scores reach +-8: the cap bites
+    out, lse = oracle.sparse_mla_fwd(q, kv, phys, scale, 512, logit_cap=cap)
+    # element-by-element restatement with math.tanh
+    for t in range(T):
+        for h in range(H):
+            sc, rows = [], []
+            for j in range(K):
+                if phys[t, j] < 0:
+                    continue
+                dot = sum(float(q[t, h, d]) * float(kv[phys[t, j], d]) for d in range(D)) * scale
+                sc.append(cap * math.tanh(dot / cap))
+                rows.append(kv[phys[t, j], :512])
+            m = max(sc)
+            w = [math.exp(x - m) for x in sc]
+            tot = sum(w)
+            assert abs(lse[t, h] - (m + math.log(tot))) < 1e-12
+            want = sum(wi / tot * r for wi, r in zip(w, rows))
+            assert np.abs(out[t, h] - want).max() < 1e-12
+    assert (lse <= cap + math.log(K) + 1e-12).all()       # every capped score is below cap
+    raw_out, raw_lse = oracle.sparse_mla_fwd(q, kv, phys, scale, 512)
+    assert np.abs(lse - raw_lse).max() > 0.5              # ... and the cap changed the result
+    big_out, big_lse = oracle.sparse_mla_fwd(q, kv, phys, scale, 512, logit_cap=1e6)
+    assert np.abs(big_lse - raw_lse).max() < 1e-9 and np.abs(big_out - raw_out).max() < 1e-9
+    # all keys equal: every score is s, so lse = cap tanh(s / cap) + log n and out = v
+    kv_same = np.tile(kv[:1], (N, 1))
+    o2, l2 = oracle.sparse_mla_fwd(q, kv_same, phys[:, :8].clip(min=0), scale, 512, logit_cap=cap)
+    s_raw = (q @ kv_same[0]) * scale
+    assert np.abs(l2 - (cap * np.tanh(s_raw / cap) + math.log(8))).max() < 1e-12
+    assert np.abs(o2 - kv_same[0, :512]).max() < 1e-12
