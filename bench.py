@@ -22,6 +22,11 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+TRAFFIC_NOTE = ("replayed from profiles/hbm_traffic.json (separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of the "
+                "same command, see profiles/*.md for the build they were taken on); not counted in this run")
+TIMING_NOTE = ("value and ms_per_step: wall clock over the timed steps, Python launch overhead included; "
+               "roofline.achieved and kernel_ms: one HIP event pair on the launch stream around the same steps; "
+               "steps rotate over independent input sets instead of flushing the caches between launches")
 
 
 def parse():
@@ -52,33 +57,50 @@ def measured_traffic(workload):
         return None
 
 
-def cpu_baseline(cfg, n_seq):
-    """numpy oracle (fp32, BLAS threads = host cores) on the first n_seq sequences of the workload."""
+def _time_oracle(qn, kv_small, phys_small, sm_scale):
+    """Median time of the numpy oracle (fp32, BLAS threads = host cores) on the given sample: at
+    least 3 runs, then more until about 10 s of CPU time are spent.  Returns (TFLOP/s, runs)."""
     import numpy as np
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle
+    n_valid = int((phys_small >= 0).sum())
+    flops = 2.0 * n_valid * qn.shape[1] * (576 + 512)
+    oracle.sparse_mla_fwd(qn[:1], kv_small, phys_small[:1], sm_scale, 512, dtype=np.float32)
+    reps, t_used, times = 0, 0.0, []
+    while reps < 3 or (t_used < 10.0 and reps < 50):
+        t0 = time.perf_counter()
+        oracle.sparse_mla_fwd(qn, kv_small, phys_small, sm_scale, 512, dtype=np.float32)
+        dt = time.perf_counter() - t0
+        times.append(dt)
+        t_used += dt
+        reps += 1
+    times.sort()
+    return flops / times[len(times) // 2] / 1e12, reps
+
+
+def cpu_baseline(cfg, n_seq):
+    """The oracle on the first n_seq sequences of a decode workload."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
     from _util import oracle_inputs
     sub = dict(cfg)
     sub["q"], sub["indices"] = cfg["q"][:n_seq], cfg["indices"][:n_seq]
     if cfg["block_table"] is not None:
         sub["block_table"] = cfg["block_table"][:n_seq]
     qn, kv_small, phys_small, _ = oracle_inputs(sub)
-    n_valid = int((phys_small >= 0).sum())
-    H = qn.shape[1]
-    flops = 2.0 * n_valid * H * (576 + 512)
-    oracle.sparse_mla_fwd(qn[:1], kv_small, phys_small[:1], cfg["sm_scale"], 512, dtype=np.float32)
-    reps, t_used = 0, 0.0
-    best = []
-    while reps < 3 or (t_used < 10.0 and reps < 50):
-        t0 = time.perf_counter()
-        oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfg["sm_scale"], 512, dtype=np.float32)
-        dt = time.perf_counter() - t0
-        best.append(dt)
-        t_used += dt
-        reps += 1
-    best.sort()
-    med = best[len(best) // 2]
-    return flops / med / 1e12, reps
+    return _time_oracle(qn, kv_small, phys_small, cfg["sm_scale"])
+
+
+def cpu_baseline_prefill(cfg, n_rows=256):
+    """The oracle on every (tokens / n_rows)-th query token of the causal prefill (a stratified
+    sample: short and long index lists in the workload's own proportion)."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from _util import oracle_inputs
+    T = cfg["q"].shape[1]
+    pick = list(range(T // n_rows - 1, T, T // n_rows))
+    sub = dict(cfg)
+    sub["q"] = cfg["q"][0, pick]                                   # [n_rows, H, 576]
+    sub["indices"] = cfg["indices"][0, pick]
+    qn, kv_small, phys_small, _ = oracle_inputs(sub)
+    return _time_oracle(qn, kv_small, phys_small, cfg["sm_scale"]) + (len(pick),)
 
 
 def main():
@@ -130,6 +152,17 @@ def main():
         s["q"], s["indices"] = q, idx.view(B, 1, K).to(dev)
         sets.append(s)
 
+    # the same index sets with their padding moved to the end of every list (the benchmark
+    # shuffles padding through the list; both orders are reported for the bf16 decode)
+    tail_sets = []
+    if a.workload == "decode_bf16":
+        for c in sets:
+            idx = c["indices"]
+            order = torch.argsort((idx < 0).to(torch.int8), dim=-1, stable=True)
+            t = dict(c)
+            t["indices"] = torch.gather(idx, -1, order).contiguous()
+            tail_sets.append(t)
+
     T = cfg["q"].shape[0] * cfg["q"].shape[1]
     H = cfg["q"].shape[2]
     K = cfg["indices"].shape[-1]
@@ -138,8 +171,9 @@ def main():
     ws_bytes = lib.smla_workspace_bytes(T, H, 512, n_splits)
     ws = ft.make_workspace(ws_bytes, dev) if ws_bytes else None
 
-    def step(i):
-        c = sets[i % len(sets)]
+    def step(i, which=None):
+        which = which or sets
+        c = which[i % len(which)]
         return ft.sparse_mla_fwd(c["q"], c["kv_cache"], c["indices"], c["sm_scale"], 512,
                                  block_table=c["block_table"], page_size=c["page_size"], kv_format=fmt,
                                  n_splits=n_splits, workspace=ws)
@@ -170,6 +204,18 @@ def main():
     torch.cuda.synchronize()
     op_ms = sorted(x.elapsed_time(y) for x, y in ev)
     op_ms_avg = sum(op_ms) / len(op_ms)
+    tail_ms = None
+    if tail_sets:
+        for i in range(min(a.warmup, 10)):
+            step(i, tail_sets)
+        torch.cuda.synchronize()
+        f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        f0.record()
+        for i in range(a.steps):
+            step(i, tail_sets)
+        f1.record()
+        torch.cuda.synchronize()
+        tail_ms = f0.elapsed_time(f1) / a.steps
 
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     gbs = nbytes / (ms_per_step * 1e-3) / 1e9
@@ -180,6 +226,7 @@ def main():
         roof = dict(bound="mfma", achieved=flops / (kern_ms * 1e-3) / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = measured_traffic(a.workload)
+    roof["traffic_source"] = TRAFFIC_NOTE
     roof["kernel"] = "fwd_tall_kernel" if H > 32 else "fwd_short_kernel"
     roof["kernel_ms"] = kern_ms
     roof["other_bound"] = (dict(bound="hbm", achieved=nbytes / (kern_ms * 1e-3) / 1e9, peak=PEAK_HBM_GBS, unit="GB/s")
@@ -206,7 +253,20 @@ def main():
         "event_ms_per_launch": {"avg": op_ms_avg, "p50": op_ms[len(op_ms) // 2], "p20": op_ms[len(op_ms) // 5],
                               "p80": op_ms[(4 * len(op_ms)) // 5]},
         "roofline": roof,
+        "timing": TIMING_NOTE,
     }
+    if tail_ms is not None:
+        res["padding_order"] = {"shuffled_kernel_ms": kern_ms, "tail_kernel_ms": tail_ms,
+                                "note": "same index sets, -1 entries spread through the list (the headline) / moved to its end"}
+    if not a.no_cpu_baseline and a.workload == "prefill_causal_bf16":
+        try:
+            v, reps, n_rows = cpu_baseline_prefill(cfg)
+            res["cpu_baseline"] = {"value": v, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+                                   "sample": f"numpy fp32 oracle on a stratified sample of {n_rows} of the {cfg['q'].shape[1]} query "
+                                             f"tokens (every {cfg['q'].shape[1] // n_rows}th), median of {reps} runs; a rate, not extrapolated"}
+        except Exception as e:
+            res["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+                                   "sample": f"failed: {e}"}
     if not a.no_cpu_baseline and a.workload != "prefill_causal_bf16":
         n_seq = a.cpu_sample or min(cfg["q"].shape[0], 8)
         try:
@@ -249,7 +309,7 @@ def bench_gemm(a, torch, ft, workloads, dev):
         "config": {"workload": "gemm_rs_shard", "m": M, "n": N, "k": Kd, "n_chunks": cfg["n_chunks"]},
         "roofline": {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": ach / PEAK_BF16_TFLOPS, "traffic": measured_traffic("gemm_rs_shard"),
-                     "kernel": "gemm_rs_big_kernel",
+                     "traffic_source": TRAFFIC_NOTE, "kernel": "gemm_rs_big_kernel",
                      "kernel_ms": kern_ms}}
     if not a.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -299,7 +359,7 @@ def bench_kv_write(a, torch, ft, dev):
         "vs_baseline": None, "dtype": "u8" if fmt != "bf16" else "bf16", "data": "synthetic",
         "config": {"workload": a.workload, "rows": n, "pool_rows": pool_rows, "kv_format": fmt, "bytes_per_step": nbytes},
         "roofline": {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
-                     "traffic": measured_traffic(a.workload),
+                     "traffic": measured_traffic(a.workload), "traffic_source": TRAFFIC_NOTE,
                      "kernel": "quantize_kernel" if fmt != "bf16" else "kv_copy_kernel", "kernel_ms": kern_ms}}
     if not a.no_cpu_baseline:
         import numpy as np
@@ -342,7 +402,7 @@ def bench_dense(a, torch, ft, workloads, dev):
     ms = (time.perf_counter() - t0) * 1e3 / a.steps
     kern_ms = e0.elapsed_time(e1) / a.steps
     ach = flops / (kern_ms * 1e-3) / 1e12
-    print(json.dumps({
+    res = {
         "metric": "dense MLA decode TFLOP/s", "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -350,9 +410,26 @@ def bench_dense(a, torch, ft, workloads, dev):
                    "flops_per_step": flops, "bytes_per_step": nbytes},
         "roofline": {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": ach / PEAK_BF16_TFLOPS, "traffic": measured_traffic("decode_dense_bf16"),
-                     "kernel": "fwd_tall_kernel", "kernel_ms": kern_ms,
+                     "traffic_source": TRAFFIC_NOTE, "kernel": "fwd_tall_kernel", "kernel_ms": kern_ms,
                      "other_bound": {"bound": "hbm", "achieved": nbytes / (kern_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                                     "unit": "GB/s", "frac": nbytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}}}))
+                                     "unit": "GB/s", "frac": nbytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}},
+        "timing": TIMING_NOTE}
+    if not a.no_cpu_baseline:
+        n_seq = a.cpu_sample or 4
+        try:
+            idx = torch.arange(ctx, dtype=torch.int32, device=dev).repeat(n_seq, 1).view(n_seq, 1, ctx)
+            sub = dict(cfg, q=cfg["q"][:n_seq], indices=idx, block_table=bt[:n_seq])
+            sys.path.insert(0, os.path.join(ROOT, "tests"))
+            from _util import oracle_inputs
+            qn, kv_small, phys_small, _ = oracle_inputs(sub)
+            v, reps = _time_oracle(qn, kv_small, phys_small, cfg["sm_scale"])
+            res["cpu_baseline"] = {"value": v, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+                                   "sample": f"numpy fp32 oracle on the first {n_seq} of {B} sequences of the same workload, "
+                                             f"median of {reps} runs"}
+        except Exception as e:
+            res["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+                                   "sample": f"failed: {e}"}
+    print(json.dumps(res))
 
 
 def bench_topk(a, torch, ft, dev):
@@ -381,7 +458,8 @@ def bench_topk(a, torch, ft, dev):
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": a.workload, "rows": rows, "cols": n, "k": k, "bytes_per_step": nbytes},
         "roofline": {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
-                     "traffic": measured_traffic(a.workload), "kernel": "topk_resident_kernel", "kernel_ms": kern_ms}}
+                     "traffic": measured_traffic(a.workload), "traffic_source": TRAFFIC_NOTE,
+                     "kernel": "topk_resident_kernel", "kernel_ms": kern_ms}}
     if not a.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         import oracle
