@@ -13,6 +13,7 @@ from flagtree_amd import _lib as product_lib
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 _lib = None
+_keep_alive = []
 
 
 def lib():
@@ -57,7 +58,7 @@ def workspace_status(ws):
     return rc, status.value
 
 
-def forward(cfg, n_splits=1, workspace=None, dense_lens=None, scalar=False, logit_cap=0.0):
+def forward(cfg, n_splits=1, workspace=None, dense_lens=None, scalar=False, logit_cap=0.0, guard_outputs=None):
     """cfg as flagtree_amd.workloads builds it, on the CPU.  Returns (out [T, H, 512], lse [T, H], rc)."""
     l = lib()
     q = cfg["q"]
@@ -75,6 +76,10 @@ def forward(cfg, n_splits=1, workspace=None, dense_lens=None, scalar=False, logi
     fmt = _FORMATS[cfg["kv_format"]]
     out = torch.full((T, H, 512), float("nan"), dtype=q.dtype)
     lse = torch.full((T, H), float("nan"), dtype=torch.float32)
+    if guard_outputs is not None:                       # outputs between inaccessible pages (kept alive by the tensors' buffers)
+        g_out, g_lse = Guarded(out, guard_outputs), Guarded(lse, guard_outputs)
+        out, lse = g_out.tensor, g_lse.tensor
+        _keep_alive.extend([g_out, g_lse])
     btc = bt.contiguous() if bt is not None else None
     bt_ptr = btc.data_ptr() if btc is not None else None
     bt_stride = btc.shape[1] if btc is not None else 0
@@ -100,3 +105,39 @@ def forward(cfg, n_splits=1, workspace=None, dense_lens=None, scalar=False, logi
                         T, S, H, idx.shape[1], 576, 512, cfg["page_size"], bt_stride, stride, kv2.shape[0], sm,
                         n_splits, ws_ptr, ws_n, None)
     return out, lse, rc
+
+
+# ---- guarded buffers: memory the emulated kernels must not step outside of -------------------
+import mmap as _mmap
+
+_PAGE = _mmap.PAGESIZE
+_libc = ctypes.CDLL(None, use_errno=True)
+_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+
+
+class Guarded:
+    """A copy of `tensor` whose last byte sits right before an inaccessible page (``end=True``) or
+    whose first byte right after one: an emulated kernel that reads or writes past that edge of
+    the buffer dies with SIGSEGV instead of silently touching a neighbour.  (A real GPU would take
+    a memory access fault, or worse, not take one.)"""
+
+    def __init__(self, tensor, end=True):
+        t = tensor.contiguous()
+        n = t.numel() * t.element_size()
+        body = (n + _PAGE - 1) // _PAGE * _PAGE
+        self._map = _mmap.mmap(-1, body + 2 * _PAGE)
+        base = ctypes.addressof(ctypes.c_char.from_buffer(self._map))
+        for off in (0, _PAGE + body):
+            if _libc.mprotect(base + off, _PAGE, 0) != 0:
+                raise OSError(ctypes.get_errno(), "mprotect")
+        start = _PAGE + (body - n if end else 0)
+        if end and (base + start) % 16:                   # keep the 16-byte alignment the C ABI asks for
+            start -= (base + start) % 16
+        self._buf = (ctypes.c_char * n).from_buffer(self._map, start)
+        self.tensor = torch.frombuffer(self._buf, dtype=torch.uint8).view(t.dtype).view(t.shape)
+        self.tensor.copy_(t)
+
+    def close(self):
+        """Drop this object's references; the mapping goes away with the last tensor that views it."""
+        self.tensor = None
+        self._buf = None

@@ -337,3 +337,33 @@ def test_local_gemm(m, n, k, chunks):
         want = oracle.gemm_rs_local(to_np(x), to_np(w), to_np(partial), n_chunks=chunks).reshape(m, n)
         assert max_abs(to_np(out), want) <= 1e-2 + 1e-2 * float(np.abs(want).max())
     harness.configure()
+
+
+# ---- memory safety: every buffer between inaccessible pages ------------------------------------
+
+def test_no_entry_point_touches_memory_outside_its_buffers():
+    """tests/emu/guarded_cases.py runs every entry point with each input, output and workspace
+    ending right before (then starting right after) an inaccessible page; an emulated kernel that
+    reads or writes outside a buffer ends that process with SIGSEGV."""
+    import subprocess
+    script = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emu", "guarded_cases.py")
+    r = subprocess.run([sys.executable, script], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), (r.returncode, r.stdout[-1500:], r.stderr[-1500:])
+
+
+def test_guard_pages_do_catch_a_stray_access():
+    """Negative control for the test above: the same set-up with a lie about a buffer's size dies."""
+    import subprocess
+    code = (
+        "import sys, torch\n"
+        f"sys.path[:0] = [{os.path.dirname(os.path.dirname(os.path.abspath(__file__)))!r}, "
+        f"{os.path.dirname(os.path.abspath(__file__))!r}, {os.path.join(os.path.dirname(os.path.abspath(__file__)), 'emu')!r}]\n"
+        "import harness\n"
+        "kv = harness.Guarded(torch.zeros((8, 576), dtype=torch.int16), True).tensor\n"
+        "idx = torch.tensor([[7, 8]], dtype=torch.int32)\n"
+        "phys = torch.zeros((1, 2), dtype=torch.int32); rows = torch.zeros((1, 2, 576), dtype=torch.int16)\n"
+        "harness.lib().smla_gather_rows(kv.data_ptr(), 1152, idx.data_ptr(), None, phys.data_ptr(), rows.data_ptr(), "
+        "1, 1, 2, 64, 0, 0, 16, None)\n"
+        "print('survived')\n")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600)
+    assert r.returncode == -11 and "survived" not in r.stdout, (r.returncode, r.stdout, r.stderr[-500:])
