@@ -235,38 +235,23 @@ __device__ __forceinline__ g_bf16x4 g_lds_tr(uint32_t a) {
   return hw::lds_read_tr16_b64(a);
 }
 
-__global__ __launch_bounds__(1024)
-void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
-                        const float* __restrict__ partial, uint16_t* __restrict__ out, int M, int N, int K,
-                        int rows_per_chunk, long long chunk_stride) {
-  __shared__ __attribute__((aligned(1024))) uint8_t s_buf[2][kStage2];
-
+// One output tile of 128 MI rows x 256 columns (MI = 2: the full 256 x 256 tile; MI = 1: its upper
+// or lower half, used to fill the last, partly occupied round of tiles, see launch_gemm_rs).
+// Wavefront (wm, wn) owns rows 32 MI wm .. + 32 MI - 1 and columns 64 wn .. + 63.
+template <int MI>
+__device__ __forceinline__ void gemm_big_tile(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                              const float* __restrict__ partial, uint16_t* __restrict__ out, int N, int K,
+                                              int rows_per_chunk, long long chunk_stride, int m0, int n0,
+                                              uint8_t* s_buf0) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 2, wn = wave & 3;              // wave tile origin (64 * wm, 64 * wn)
+  const int wm = wave >> 2, wn = wave & 3;
   const int g = lane >> 5, c32 = lane & 31, l16 = lane & 15;
+  const uint32_t lds0 = hw::lds_addr(s_buf0);
 
-  // tile mapping: XCD x owns m-tiles [x * mt/8, (x+1) * mt/8) when mt divides by 8
-  const int mt = M / kBM2, nt = N / kBN2;
-  int tile_m, tile_n;
-  {
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    if (mt % 8 == 0) {
-      const int band = mt / 8;
-      tile_m = xcd * band + local % band;
-      tile_n = local / band;
-    } else {
-      tile_m = blockIdx.x % mt;
-      tile_n = blockIdx.x / mt;
-    }
-  }
-  if (tile_m >= mt || tile_n >= nt) return;
-  const int m0 = tile_m * kBM2, n0 = tile_n * kBN2;
-  const uint32_t lds0 = hw::lds_addr(&s_buf[0][0]);
-
-  // ---- DMA of one K-step: 32 instructions for the X tile (8 rows each) and 32 for the W tile (2
-  // rows each), 8 + 8 per wavefront.  Instruction i = 8 wave + t; the swizzles depend on i's parity
-  // only, so a lane needs two byte offsets per tile.
+  // ---- DMA of one K-step: 16 MI instructions for the X tile (8 rows each) and 32 for the W tile (2
+  // rows each), MI + 2 per wavefront.  X instruction i = MI wave + d, W instruction i = 2 wave + d;
+  // the swizzles depend on i's parity only, so a lane needs two byte offsets per tile.
   uint32_t a_off[2], b_off[2];
   {
     const int p = lane & 7, rl = lane >> 3;             // X: chunk position, row within the instruction's 8
@@ -282,14 +267,16 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
       b_off[odd] = (uint32_t)((kl * N + n0 + 8 * (4 * blk + (pb & 3))) * 2);
     }
   }
-  // DMA instruction d = 0..3 of this wavefront for the K-step at k0 into buffer buf (0, 1: X, 2, 3: W)
+  // DMA slot d = 0..3 of this wavefront for the K-step at k0 into buffer buf (0, 1: X, 2, 3: W)
   auto issue_dma = [&](int d, int k0, int buf) {
     const uint32_t dst = lds0 + buf * kStage2;
     if (d < 2) {
-      const int i = 2 * wave + d;
-      const uint64_t sa = (uint64_t)(uintptr_t)x + ((uint64_t)(m0 + 8 * i) * K + k0) * 2;
-      const uint32_t ma = dst + i * 1024;
-      hw::dma_b128(a_off[d & 1], sa, ma);
+      if (d < MI) {
+        const int i = MI * wave + d;
+        const uint64_t sa = (uint64_t)(uintptr_t)x + ((uint64_t)(m0 + 8 * i) * K + k0) * 2;
+        const uint32_t ma = dst + i * 1024;
+        hw::dma_b128(a_off[i & 1], sa, ma);
+      }
     } else {
       const int i = 2 * wave + d - 2;
       const uint64_t sb = (uint64_t)(uintptr_t)w + (uint64_t)(k0 + 2 * i) * N * 2;
@@ -298,16 +285,16 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
     }
   };
 
-  g_f32x16 acc[2][2];
+  g_f32x16 acc[MI][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // fragment addresses inside a buffer
-  const uint32_t a_lane = (uint32_t)((64 * wm + c32) * 128);              // row of A tile i = 0; + 32 i rows
+  const uint32_t a_lane = (uint32_t)((32 * MI * wm + c32) * 128);         // row of A tile i = 0; + 32 i rows
   const uint32_t a_sw = (uint32_t)((c32 >> 1) & 7);
   const uint32_t b_lane = (uint32_t)(kA2Bytes + (8 * g + (l16 >> 2)) * 512 + 32 * ((lane >> 4) & 1) + 8 * (l16 & 3));
   const uint32_t b_sw = (uint32_t)((l16 >> 2) & 3);
@@ -315,9 +302,9 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
   const int n_k = K / kBK;
 #pragma unroll
   for (int d = 0; d < 4; ++d) issue_dma(d, 0, 0);
-  auto load_frags = [&](uint32_t buf, int ks, g_bf16x8 (&af)[2], g_bf16x8 (&bf)[2]) {
+  auto load_frags = [&](uint32_t buf, int ks, g_bf16x8 (&af)[MI], g_bf16x8 (&bf)[2]) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) af[i] = g_lds_b128(buf + a_lane + i * (32 * 128) + (((2 * ks + g) ^ a_sw) << 4));
+    for (int i = 0; i < MI; ++i) af[i] = g_lds_b128(buf + a_lane + i * (32 * 128) + (((2 * ks + g) ^ a_sw) << 4));
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const uint32_t bp = buf + b_lane + (16 * ks) * 512 + (((2 * wn + j) ^ b_sw) << 6);
@@ -332,14 +319,14 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
     const uint32_t buf = lds0 + (kt & 1) * kStage2;
     const bool more = kt + 1 < n_k;
     const int k_next = (kt + 1) * kBK, buf_next = (kt + 1) & 1;
-    g_bf16x8 af[2][2], bf[2][2];
+    g_bf16x8 af[2][MI], bf[2][2];
     load_frags(buf, 0, af[0], bf[0]);
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
       if (ks + 1 < kBK / 16) load_frags(buf, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
       if (more) issue_dma(ks, k_next, buf_next);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
@@ -349,15 +336,15 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
 
   // ---- epilogue: a wavefront parks 32 rows x 64 columns (one row of its MFMA tiles) in LDS and
   // reads them back four rows a pass, four consecutive columns per lane
-  float* stage = reinterpret_cast<float*>(&s_buf[0][0]) + wave * 32 * kStage2Floats;
+  float* stage = reinterpret_cast<float*>(s_buf0) + wave * 32 * kStage2Floats;
   const int col4 = 4 * l16, rsub = lane >> 4;           // this lane's 4 columns within the wave's 64, row within a pass
   const int n = n0 + 64 * wn + col4;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < MI; ++i) {
     g_f32x4 z[8];                                       // partial sums of rows 32*i + 4*p + rsub, p < 8
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
-      const int m = m0 + 64 * wm + 32 * i + 4 * p + rsub;
+      const int m = m0 + 32 * MI * wm + 32 * i + 4 * p + rsub;
       z[p] = partial ? __builtin_nontemporal_load(reinterpret_cast<const g_f32x4*>(partial + (size_t)m * N + n))
                      : g_f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -371,7 +358,7 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
       const int row = 4 * p + rsub;
-      const int m = m0 + 64 * wm + 32 * i + row;
+      const int m = m0 + 32 * MI * wm + 32 * i + row;
       const float4 v = *reinterpret_cast<const float4*>(stage + row * kStage2Floats + col4);
       const g_f32x4 zz = z[p];
       const int chunk = m / rows_per_chunk;
@@ -385,20 +372,74 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
   }
 }
 
+// Blocks [0, n_full) take whole 256 x 256 tiles; blocks from n_full on take half tiles (128 rows),
+// two consecutive blocks of an XCD the two halves of one tile.  The hardware hands out blocks in
+// id order, so the half tiles are what runs last.
+__global__ __launch_bounds__(1024)
+void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                        const float* __restrict__ partial, uint16_t* __restrict__ out, int M, int N, int K,
+                        int rows_per_chunk, long long chunk_stride, int n_full) {
+  __shared__ __attribute__((aligned(1024))) uint8_t s_buf[2][kStage2];
+
+  // tile mapping: XCD x owns m-tiles [x * mt/8, (x+1) * mt/8) when mt divides by 8
+  const int mt = M / kBM2, nt = N / kBN2;
+  const bool halves = (int)blockIdx.x >= n_full;
+  int tile_m, tile_n, half = 0;
+  {
+    int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    if (halves) {                                       // (only with the banded mapping; n_full is a multiple of 8)
+      const int j = (int)blockIdx.x - n_full;
+      xcd = j & 7;
+      half = (j >> 3) & 1;
+      local = (n_full >> 3) + (j >> 4);
+    }
+    if (mt % 8 == 0) {
+      const int band = mt / 8;
+      tile_m = xcd * band + local % band;
+      tile_n = local / band;
+    } else {
+      tile_m = blockIdx.x % mt;
+      tile_n = blockIdx.x / mt;
+    }
+  }
+  if (tile_m >= mt || tile_n >= nt) return;
+  const int n0 = tile_n * kBN2;
+  if (halves)
+    gemm_big_tile<1>(x, w, partial, out, N, K, rows_per_chunk, chunk_stride, tile_m * kBM2 + 128 * half, n0, &s_buf[0][0]);
+  else
+    gemm_big_tile<2>(x, w, partial, out, N, K, rows_per_chunk, chunk_stride, tile_m * kBM2, n0, &s_buf[0][0]);
+}
+
+// How many of the 256 x 256 tiles are computed whole; the rest, the last and only partly filled
+// round of tiles on `n_cu` compute units, is split into half tiles when that fills the round:
+// 896 tiles on 256 units are 3 rounds + 128 tiles, which as 256 half tiles keep every unit busy for
+// 3/4 of a round (a half tile moves 3/4 of a tile's bytes into LDS) instead of half the units for a
+// whole one.
+int gemm_full_tiles(int mt, int nt, int n_cu) {
+  const long long tiles = (long long)mt * nt;
+  if (mt % 8 != 0 || n_cu <= 0) return (int)tiles;
+  const long long rest = tiles % n_cu;
+  return rest > 0 && 2 * rest <= n_cu ? (int)(tiles - rest) : (int)tiles;
+}
+
 int launch_gemm_rs(const void* x, const void* w, const float* partial, void* out, int m, int n, int k,
-                   int n_chunks, int64_t chunk_stride, hipStream_t s) {
+                   int n_chunks, int64_t chunk_stride, int n_cu, hipStream_t s) {
   if (m % kBM != 0 || n % kBN != 0 || k % kBK != 0) return SMLA_EINVAL_SHAPE;
   // the DMA's per-lane byte offsets are 32-bit
   const bool big = m % kBM2 == 0 && (long long)8 * k * 2 < (1ll << 31) && ((long long)2 * n + n) * 2 < (1ll << 31);
   const int bm = big ? kBM2 : kBM;
   const int mt = m / bm, nt = n / kBN;
-  const long long blocks = (long long)((mt + 7) / 8 * 8) * nt;
-  if (blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
-  if (big)
-    hipLaunchKernelGGL(gemm_rs_big_kernel, dim3((unsigned)blocks), dim3(1024), 0, s, 
+  long long blocks = (long long)((mt + 7) / 8 * 8) * nt;
+  if (blocks > 0x3fffffffLL) return SMLA_EINVAL_SHAPE;
+  if (big) {
+    const long long tiles = (long long)mt * nt;
+    long long n_full = gemm_full_tiles(mt, nt, n_cu);
+    if (n_full < tiles) blocks = n_full + 2 * (tiles - n_full);   // (only with mt a multiple of 8: blocks was mt * nt)
+    else n_full = blocks;                                         // no half tiles
+    hipLaunchKernelGGL(gemm_rs_big_kernel, dim3((unsigned)blocks), dim3(1024), 0, s,
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), partial, static_cast<uint16_t*>(out), m, n, k,
-        m / n_chunks, (long long)chunk_stride);
-  else
+        m / n_chunks, (long long)chunk_stride, (int)n_full);
+  } else
     hipLaunchKernelGGL(gemm_rs_kernel, dim3((unsigned)blocks), dim3(256), 0, s, 
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), partial, static_cast<uint16_t*>(out), m, n, k,
         m / n_chunks, (long long)chunk_stride);

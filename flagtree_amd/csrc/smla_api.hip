@@ -285,7 +285,7 @@ int smla_gemm_rs_local(const void* x, const void* w, const float* partial, void*
   if (!aligned16(x) || !aligned16(w) || !aligned16(out) || (partial && !aligned16(partial)) ||
       (chunk_stride % 8) != 0)
     return SMLA_EINVAL_ALIGN;
-  return launch_gemm_rs(x, w, partial, out, m, n, k, n_chunks, chunk_stride,
+  return launch_gemm_rs(x, w, partial, out, m, n, k, n_chunks, chunk_stride, device_cus(),
                         static_cast<hipStream_t>(stream));
 }
 

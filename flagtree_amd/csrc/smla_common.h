@@ -210,7 +210,7 @@ int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_
 int launch_zero(void* ptr, size_t bytes, hipStream_t s);
 int launch_workspace_init(void* workspace, hipStream_t s);
 int launch_gemm_rs(const void* x, const void* w, const float* partial, void* out, int m, int n,
-                   int k, int n_chunks, int64_t chunk_stride, hipStream_t s);
+                   int k, int n_chunks, int64_t chunk_stride, int n_cu, hipStream_t s);
 
 inline int hip_status(hipError_t e) { return e == hipSuccess ? SMLA_OK : SMLA_EHIP_BASE - (int)e; }
 

@@ -87,6 +87,7 @@ const std::function<void()>* g_body = nullptr;
 int g_dma_eager = 0;
 unsigned g_order_seed = 0;
 unsigned long long g_launches = 0;
+int g_cu_count = 256;
 std::vector<char*> g_stacks;
 
 void yield() { emu_switch(&g_cur->sp, g_sched_sp); }
@@ -197,6 +198,7 @@ Lane* self() { return &g_cur->lane; }
 Dim3 block_idx() { return g_block_idx; }
 Dim3 block_dim() { return g_block_dim; }
 Dim3 grid_dim() { return g_grid_dim; }
+int cu_count() { return g_cu_count; }
 
 int wave_rendezvous(const void* post, size_t bytes, uint32_t tag) {
   Fiber* f = g_cur;
@@ -298,4 +300,5 @@ extern "C" {
 void emu_set_dma_mode(int eager) { emu::g_dma_eager = eager; }
 void emu_set_block_order(unsigned seed) { emu::g_order_seed = seed; }
 unsigned long long emu_launch_count(void) { return emu::g_launches; }
+void emu_set_cu_count(int n) { emu::g_cu_count = n; }
 }

@@ -56,6 +56,7 @@ void dma_issue(const void* src, uint32_t lds_dst, int bytes);
 void dma_wait(int allowed_in_flight);
 
 void launch(Dim3 grid, Dim3 block, const std::function<void()>& body);
+int cu_count();                       // what the stand-in device reports as its number of compute units
 
 [[noreturn]] void fail(const char* fmt, ...);
 
@@ -66,4 +67,5 @@ extern "C" {
 void emu_set_dma_mode(int eager);        // 0: moves land at the wait (default), 1: at issue
 void emu_set_block_order(unsigned seed); // 0: ascending block ids, else a seeded shuffle
 unsigned long long emu_launch_count(void);
+void emu_set_cu_count(int n);            // before the library's first query (it caches the answer); default 256
 }

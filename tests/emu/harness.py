@@ -14,6 +14,7 @@ from flagtree_amd import _lib as product_lib
 HERE = os.path.dirname(os.path.abspath(__file__))
 _lib = None
 _keep_alive = []
+EMU_CUS = 16      # compute units the stand-in device reports: small, so that small shapes reach the planning corner cases
 
 
 def lib():
@@ -31,6 +32,8 @@ def lib():
         l.emu_set_dma_mode.argtypes = [ctypes.c_int]
         l.emu_set_block_order.argtypes = [ctypes.c_uint]
         l.emu_launch_count.restype = ctypes.c_ulonglong
+        l.emu_set_cu_count.argtypes = [ctypes.c_int]
+        l.emu_set_cu_count(EMU_CUS)                      # before the library's first (cached) query
         _lib = l
     return _lib
 

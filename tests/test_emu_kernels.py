@@ -322,7 +322,9 @@ def test_topk_indices_exact(rows, n, k):
     assert np.array_equal(to_np(out), oracle.topk_indices(to_np(scores), k, to_np(lens)))
 
 
-@pytest.mark.parametrize("m,n,k,chunks", [(256, 256, 128, 2), (128, 512, 192, 1), (384, 256, 64, 3), (512, 256, 128, 4)])
+@pytest.mark.parametrize("m,n,k,chunks", [(256, 256, 128, 2), (128, 512, 192, 1), (384, 256, 64, 3), (512, 256, 128, 4),
+                                          (2048, 256, 64, 8),      # 8 tiles on 16 units: every tile as two half tiles
+                                          (2048, 768, 128, 2)])    # 24 tiles: 16 whole + 8 split into 16 half tiles
 def test_local_gemm(m, n, k, chunks):
     g = torch.Generator().manual_seed(m + n + k)
     x = (torch.randn((m, k), generator=g) * 0.1).to(torch.bfloat16)
