@@ -43,6 +43,8 @@ def parse():
                     help="first run three plain 1 GiB device copies (known HBM traffic) so a rocprofv3 --pmc "
                          "run of this command holds a reference kernel to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
+    ap.add_argument("--few-fp8", action="store_true",
+                    help="decode_fp8 on the two-workgroups-per-CU kernel (sets FLAGTREE_SMLA_FEW_FP8=1; opt-in until measured)")
     return ap.parse_args()
 
 
@@ -109,6 +111,8 @@ def main():
         print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported in this build "
               "(no collective path exists: work units are independent per token).", file=sys.stderr)
         sys.exit(2)
+    if a.few_fp8:
+        os.environ["FLAGTREE_SMLA_FEW_FP8"] = "1"
     import torch
     import flagtree_amd as ft
     from flagtree_amd import workloads
@@ -227,7 +231,7 @@ def main():
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = measured_traffic(a.workload)
     roof["traffic_source"] = TRAFFIC_NOTE
-    roof["kernel"] = "fwd_tall_kernel" if H > 32 else "fwd_short_kernel"
+    roof["kernel"] = "fwd_tall_kernel" if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
     roof["kernel_ms"] = kern_ms
     roof["other_bound"] = (dict(bound="hbm", achieved=nbytes / (kern_ms * 1e-3) / 1e9, peak=PEAK_HBM_GBS, unit="GB/s")
                            if not hbm_bound else

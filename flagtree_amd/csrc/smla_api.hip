@@ -1,6 +1,8 @@
 // C ABI of libflagtree_smla.so: argument validation and kernel dispatch.
 #include "smla_common.h"
 
+#include <stdlib.h>
+
 using namespace smla;
 
 namespace {
@@ -21,6 +23,14 @@ int check_common(const void* q, const void* kv, const int32_t* indices, const vo
   if (!aligned16(q) || !aligned16(kv) || !aligned16(out)) return SMLA_EINVAL_ALIGN;
   if ((reinterpret_cast<uintptr_t>(indices) & 3u) != 0) return SMLA_EINVAL_ALIGN;   // read 4 bytes at a time
   return SMLA_OK;
+}
+
+// Kernels that have passed the parity checks but whose speed has not been measured on hardware
+// yet stay behind a switch until it has: FLAGTREE_SMLA_FEW_FP8=1 sends few-heads launches over an
+// fp8 cache to the two-workgroups-per-CU kernel (smla_mfma_few_fp8.hip).  Read at every call.
+bool few_fp8_enabled() {
+  const char* e = getenv("FLAGTREE_SMLA_FEW_FP8");
+  return e != nullptr && e[0] == '1';
 }
 
 int device_cus() {
@@ -103,7 +113,9 @@ int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t t
   if (kv_format == SMLA_KV_F32) return 1;
   // one 4-wave workgroup per CU is resident at a time; each covers 64 (or, for <= 32 heads, 16)
   // heads of one token
-  const int slots = device_cus();
+  // (the opt-in fp8 kernel keeps two workgroups per CU, and wants a few more than that so their phases drift apart)
+  const bool few_fp8 = kv_format == SMLA_KV_FP8_B128 && n_heads <= 32 && few_fp8_enabled();
+  const int slots = few_fp8 ? 4 * device_cus() : device_cus();
   const int per_wg = n_heads <= 32 ? 16 : 64;
   const long long groups = (long long)n_tokens * ((n_heads + per_wg - 1) / per_wg);
   int want = (int)((slots + groups - 1) / groups);
@@ -174,7 +186,9 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
     p.part_out = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + SMLA_WS_COUNTER_BYTES);
     p.part_lse = p.part_out + (size_t)n_tokens * n_splits * n_heads * d_v;
   }
-  return n_heads <= 32 ? launch_fwd_short(kv_format, p, s) : launch_fwd_tall(kv_format, p, s);
+  if (n_heads > 32) return launch_fwd_tall(kv_format, p, s);
+  if (kv_format == SMLA_KV_FP8_B128 && few_fp8_enabled()) return launch_fwd_few_fp8(p, s);
+  return launch_fwd_short(kv_format, p, s);
 }
 
 int smla_fwd(int kv_format, const void* q, const void* kv, const int32_t* indices,

@@ -27,8 +27,11 @@ def _guard_cfg(cfg, end):
     return out, keep
 
 
-def forward_case(make, n_splits, dense=False):
+def forward_case(make, n_splits, dense=False, env=None):
     def run(end):
+        for k in ("FLAGTREE_SMLA_FEW_FP8",):
+            os.environ.pop(k, None)
+        os.environ.update(env or {})
         cfg = make()
         gcfg, keep = _guard_cfg(cfg, end)
         T = cfg["q"].numel() // (cfg["q"].shape[-2] * 576)
@@ -132,6 +135,8 @@ CASES = {
     "short_bf16_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=2, heads=16, pages_per_seq=5, topk=200, pad_frac=0.06), 2),
     "short_bf16_ragged_heads": forward_case(lambda: workloads.decode_bf16("cpu", batch=1, heads=9, pages_per_seq=5, topk=150, pad_frac=0.06), 1),
     "short_fp8_split": forward_case(lambda: fp8_cfg(2, 16, 4, 150), 2),
+    "few_fp8_split": forward_case(lambda: fp8_cfg(2, 16, 4, 150), 2, env={"FLAGTREE_SMLA_FEW_FP8": "1"}),
+    "few_fp8_ragged_heads": forward_case(lambda: fp8_cfg(1, 9, 4, 100), 1, env={"FLAGTREE_SMLA_FEW_FP8": "1"}),
     "dense_tall": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=128, pages_per_seq=3, topk=64), 2, dense=True),
     "dense_short_fp8": forward_case(lambda: fp8_cfg(3, 16, 3, 64), 1, dense=True),
     "scalar_f32": forward_case(lambda: workloads.plumbing_f32("cpu", tokens=2, heads=16, s_kv=256, topk=40), 1),

@@ -105,6 +105,69 @@ def test_fp8_records(heads, n_splits):
     _check(cfg, out, lse)
 
 
+@pytest.fixture
+def few_fp8_kernel(monkeypatch):
+    """Routes few-heads fp8 launches to the two-workgroups-per-CU kernel (opt-in until it is measured)."""
+    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
+
+
+@pytest.mark.parametrize("heads,n_splits,topk", [(16, 1, 300), (16, 2, 300), (8, 1, 70), (16, 3, 1100), (30, 2, 200), (16, 4, 40)])
+def test_fp8_records_column_split_kernel(few_fp8_kernel, heads, n_splits, topk):
+    cfg, _ = _fp8_cfg(2, heads, 20, topk, pad_frac=0.05)
+    out, lse = _forward_all_ways(cfg, n_splits)
+    _check(cfg, out, lse)
+    # it is a different kernel: same results to the bar, not to the bit
+    os.environ.pop("FLAGTREE_SMLA_FEW_FP8")
+    out1, lse1, rc = harness.forward(cfg, n_splits=n_splits)
+    assert rc == 0 and not torch.equal(out1.view(torch.int16), out.view(torch.int16))
+    assert max_abs(to_np(out1), to_np(out)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse)) <= 1e-5
+
+
+def test_column_split_kernel_edge_cases_redo_and_dense(few_fp8_kernel):
+    # edge cases: empty list, single entry, duplicates, interleaved padding, out-of-range
+    g = torch.Generator().manual_seed(7)
+    latent = (torch.randn((300, 576), generator=g) * 0.1).to(torch.bfloat16)
+    rec = torch.zeros((300, 656), dtype=torch.uint8)
+    assert harness.lib().smla_kv_quantize_fp8(latent.data_ptr(), None, rec.data_ptr(), 300, 300, None) == 0
+    q = (torch.randn((6, 16, 576), generator=g) * 0.1).to(torch.bfloat16)
+    idx = torch.full((6, 70), -1, dtype=torch.int32)
+    idx[1, 33] = 5
+    idx[2, :] = torch.randperm(300, generator=g)[:70].to(torch.int32)
+    idx[3, :35] = 17
+    idx[4, ::2] = torch.arange(35, dtype=torch.int32)
+    idx[5, 0] = 299
+    idx[5, 1] = 300
+    cfg = dict(q=q, kv_cache=rec, indices=idx, block_table=None, page_size=64, sm_scale=576 ** -0.5, kv_format="fp8_e4m3_b128")
+    for ns in (1, 2):
+        out, lse = _forward_all_ways(cfg, ns)
+        _check(cfg, out, lse)
+        assert (to_np(out)[0] == 0).all() and np.isneginf(to_np(lse)[0]).all()
+    # scores that outgrow the first tile's maximum: the exact two-pass path
+    latent = (torch.randn((400, 576), generator=g) * 4.0).to(torch.bfloat16)
+    latent[:64] *= 0.01
+    rec = torch.zeros((400, 656), dtype=torch.uint8)
+    assert harness.lib().smla_kv_quantize_fp8(latent.data_ptr(), None, rec.data_ptr(), 400, 400, None) == 0
+    q = (torch.randn((2, 16, 576), generator=g) * 4.0).to(torch.bfloat16)
+    cfg = dict(q=q, kv_cache=rec, indices=torch.arange(200, dtype=torch.int32).repeat(2, 1), block_table=None, page_size=64,
+               sm_scale=576 ** -0.5, kv_format="fp8_e4m3_b128")
+    ro, rl = run_oracle(cfg)
+    for ns in (1, 2):
+        out, lse = _forward_all_ways(cfg, ns)
+        assert max_abs(to_np(lse), rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
+        assert max_abs(to_np(out), ro) <= 1.2e-2 * max(1.0, float(np.abs(ro).max()))
+    # dense decode with a logit cap
+    cfg, _ = _fp8_cfg(3, 16, 5, 64)
+    lens = torch.tensor([300, 1, 129], dtype=torch.int32)
+    idx = torch.full((3, 1, 320), -1, dtype=torch.int32)
+    for b, n in enumerate(lens.tolist()):
+        idx[b, 0, :n] = torch.arange(n, dtype=torch.int32)
+    qn, kv_small, phys_small, _ = oracle_inputs(dict(cfg, indices=idx))
+    for cap in (0.0, 0.02):
+        wo, wl = oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfg["sm_scale"], 512, logit_cap=cap)
+        out, lse = _forward_all_ways(cfg, 2, dense_lens=lens, logit_cap=cap)
+        assert max_abs(to_np(lse), wl) <= 1e-3 and max_abs(to_np(out), wo) <= 1e-2
+
+
 def test_more_than_one_chunk_of_the_list():
     """Lists longer than the 1024 entries the kernels compact at a time, ragged last tile."""
     from flagtree_amd import workloads

@@ -664,3 +664,73 @@ def test_properties_at_full_fp8_decode_size(dev):
     assert (out[:8].float() - so.float()).abs().max().item() <= OUT_TOL
     assert (lse[:8] - sl).abs().max().item() <= LSE_TOL
     _check(dict(sub, q=sub["q"][:2], indices=sub["indices"][:2], block_table=sub["block_table"][:2]), out[:2], lse[:2])
+
+
+# ---- the two-workgroups-per-CU fp8 kernel (opt-in until it has been measured) -------------------
+
+@pytest.fixture
+def few_fp8_kernel(monkeypatch):
+    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
+
+
+@pytest.mark.parametrize("heads,n_splits,topk", [(16, 1, 512), (16, 2, 512), (8, 3, 300), (30, 2, 700), (16, None, 2048)])
+def test_column_split_fp8_kernel_against_oracle(dev, few_fp8_kernel, heads, n_splits, topk):
+    from flagtree_amd import workloads
+    cfg = workloads.decode_fp8(dev, batch=5, heads=heads, pages_per_seq=40, topk=topk, pad_frac=0.03)
+    out, lse = _fwd(cfg, n_splits=n_splits)
+    _check(cfg, out, lse)
+
+
+def test_column_split_fp8_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch):
+    """Full fp8 decode size: the two kernels agree to the bar (they sum in different orders), and a
+    slice of the batch agrees with the oracle."""
+    from flagtree_amd import workloads
+    cfg = workloads.decode_fp8(dev)
+    out0, lse0 = _fwd(cfg)
+    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
+    out1, lse1 = _fwd(cfg)
+    torch.cuda.synchronize()
+    assert not torch.equal(out0, out1)                       # it really is the other kernel
+    assert max_abs(to_np(out1), to_np(out0)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse0)) <= 1e-4
+    sub = dict(cfg, q=cfg["q"][:4], indices=cfg["indices"][:4], block_table=cfg["block_table"][:4])
+    ro, rl = run_oracle(sub)
+    assert max_abs(to_np(out1[:4]).reshape(4, 16, 512), ro) <= OUT_TOL and max_abs(to_np(lse1[:4]).reshape(4, 16), rl) <= LSE_TOL
+
+
+def test_column_split_fp8_kernel_edge_cases_and_dense(dev, few_fp8_kernel):
+    import flagtree_amd as ft
+    g = torch.Generator().manual_seed(7)
+    latent = (torch.randn((300, 576), generator=g) * 0.1).to(torch.bfloat16).to(dev)
+    rec = ft.quantize_kv_fp8(latent)
+    q = (torch.randn((6, 16, 576), generator=g) * 0.1).to(torch.bfloat16).to(dev)
+    idx = torch.full((6, 70), -1, dtype=torch.int32)
+    idx[1, 33] = 5
+    idx[2, :] = torch.randperm(300, generator=g)[:70].to(torch.int32)
+    idx[3, :35] = 17
+    idx[4, ::2] = torch.arange(35, dtype=torch.int32)
+    idx[5, 0] = 299
+    idx[5, 1] = 300
+    cfg = dict(q=q, kv_cache=rec, indices=idx.to(dev), block_table=None, page_size=64, sm_scale=576 ** -0.5,
+               kv_format="fp8_e4m3_b128")
+    for ns in (1, 2):
+        out, lse = _fwd(cfg, n_splits=ns)
+        _check(cfg, out, lse)
+        assert (to_np(out)[0] == 0).all() and np.isneginf(to_np(lse)[0]).all()
+    # dense decode with a logit cap through the same kernel
+    B, L, page_size, cap = 3, 700, 64, 0.02
+    lens = torch.tensor([L, 3, 300], dtype=torch.int32)
+    n_pages = -(-L // page_size)
+    req = torch.randperm(2 * B * n_pages, generator=g)[:B * n_pages].to(torch.int32).view(B, n_pages)
+    lat = (torch.randn((2 * B * n_pages * page_size, 576), generator=g) * 0.1).to(torch.bfloat16)
+    k_buffer = ft.quantize_kv_fp8(lat.to(dev)).view(-1, page_size, 656)
+    qd = (torch.randn((B, 16, 576), generator=g) * 0.1).to(torch.bfloat16)
+    o, lse = ft.decode_attention_fwd(qd.to(dev), k_buffer, None, None, req.to(dev), lens.to(dev), None, 2, 576 ** -0.5,
+                                     page_size, logit_cap=cap)
+    max_len = n_pages * page_size
+    idxd = torch.arange(max_len, dtype=torch.int32).repeat(B, 1)
+    idxd[idxd >= lens[:, None]] = -1
+    cfgd = {"q": qd.view(B, 1, 16, 576), "indices": idxd.view(B, 1, max_len), "kv_cache": k_buffer, "block_table": req,
+            "page_size": page_size, "kv_format": "fp8_e4m3_b128", "sm_scale": 576 ** -0.5}
+    qn, kv_small, phys_small, _ = oracle_inputs(cfgd)
+    wo, wl = oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfgd["sm_scale"], 512, logit_cap=cap)
+    assert max_abs(to_np(lse), wl.reshape(B, 16)) <= 1e-3 and max_abs(to_np(o), wo.reshape(B, 16, 512)) <= 1e-2

@@ -7,24 +7,36 @@ registers the hardware has not filled yet."""
 import os
 import re
 import subprocess
+import tempfile
 
 import pytest
 
 from flagtree_amd import build
 
 LDS_PER_CU = 160 * 1024
-# kernels that are allowed to use scratch memory: the many-heads forward over an fp8 cache
-# converts its tiles in registers next to 128 accumulators and 72 Q registers
-MAY_SPILL = ("fwd_tall_kernelILi1E",)
+# Kernels that may park registers in scratch memory OUTSIDE their inner loops (checked below):
+#  * the many-heads forward over an fp8 cache converts its tiles in registers next to 128
+#    accumulators and 72 Q registers; it parks values across its prologue,
+#  * the two-workgroups-per-CU fp8 kernel is capped at 256 registers and parks a few across the
+#    per-chunk set-up.
+MAY_SPILL = ("fwd_tall_kernelILi1E", "fwd_few_fp8_kernel")
+
+_cache = {}
 
 
-def _resource_usage(source):
+def _compile(source):
+    """(kernel name -> resource figures, assembly text) of one source file, from a single compile."""
+    if source in _cache:
+        return _cache[source]
     flags = [f for f in build.FLAGS if f not in ("-fPIC", "-shared")]
-    cmd = [build.HIPCC] + flags + ["--cuda-device-only", "-Rpass-analysis=kernel-resource-usage", "-I",
-                                   os.path.join(os.path.dirname(build.HERE), "include"),
-                                   "-c", os.path.join(build.CSRC, source), "-o", os.devnull]
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
-    assert res.returncode == 0, res.stdout[-2000:]
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, "out.s")
+        cmd = [build.HIPCC] + flags + ["--cuda-device-only", "-S", "-Rpass-analysis=kernel-resource-usage", "-I",
+                                       os.path.join(os.path.dirname(build.HERE), "include"),
+                                       os.path.join(build.CSRC, source), "-o", asm]
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900)
+        assert res.returncode == 0, res.stdout[-2000:]
+        text = open(asm).read()
     kernels, cur = {}, None
     for line in res.stdout.splitlines():
         m = re.search(r"remark: \s*Function Name: (\S+)", line)
@@ -34,18 +46,65 @@ def _resource_usage(source):
         m = re.search(r"remark: \s*([A-Za-z ]+?)(?: \[[^\]]*\])?: (\d+)", line)
         if m and cur is not None:
             cur[m.group(1).strip()] = int(m.group(2))
-    return kernels
+    _cache[source] = (kernels, text)
+    return _cache[source]
+
+
+def _resource_usage(source):
+    return _compile(source)[0]
+
+
+def _scratch_in_inner_loops(asm_text):
+    """{kernel: number of scratch loads / stores inside innermost loops}.  The compiler annotates
+    basic blocks with the loop they belong to; an innermost loop's header says 'Inner Loop Header'."""
+    out, kernel, inner, block_loop = {}, None, set(), None
+    lines = asm_text.splitlines()
+    for line in lines:                                    # first pass: the innermost loop headers
+        m = re.match(r"^(\.LBB\d+_\d+):.*This Inner Loop Header", line)
+        if m:
+            inner.add(m.group(1)[2:])                     # 'BB3_195'
+    for line in lines:
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            kernel, block_loop = m.group(1), None
+            out.setdefault(kernel, 0)
+            continue
+        if line.startswith(".Lfunc_end"):
+            kernel = None
+            continue
+        m = re.match(r"^\.L(BB\d+_\d+):(.*)", line)
+        if m:
+            label, note = m.group(1), m.group(2)
+            h = re.search(r"in Loop: Header=(BB\d+_\d+)", note)
+            block_loop = label if label in inner else (h.group(1) if h and h.group(1) in inner else None)
+            continue
+        m = re.match(r"^; %bb\.\d+:(.*)", line)          # fall-through blocks carry the same annotation
+        if m:
+            h = re.search(r"in Loop: Header=(BB\d+_\d+)", m.group(1))
+            block_loop = h.group(1) if h and h.group(1) in inner else None
+            continue
+        if kernel and block_loop and re.match(r"^\s+scratch_(load|store)", line):
+            out[kernel] += 1
+    return out
 
 
 @pytest.mark.parametrize("source", [s for s in build.SOURCES if s != "smla_api.hip"])
 def test_kernels_fit_the_cu_and_do_not_spill(source):
-    kernels = _resource_usage(source)
+    kernels, asm = _compile(source)
     assert kernels, "no kernel found in " + source
     for name, use in kernels.items():
         assert use["LDS Size"] <= LDS_PER_CU, (name, use)
         assert use["VGPRs"] <= 256 and use["AGPRs"] <= 256, (name, use)
         if not any(tag in name for tag in MAY_SPILL):
             assert use["ScratchSize"] == 0 and use["VGPRs Spill"] == 0, (name, use)
+    hot = _scratch_in_inner_loops(asm)
+    assert hot and all(n == 0 for n in hot.values()), {k: v for k, v in hot.items() if v}
+
+
+def test_two_workgroups_of_the_column_split_fp8_kernel_fit_a_cu():
+    few = _resource_usage("smla_mfma_few_fp8.hip")
+    assert few and all(u["Occupancy"] >= 2 and u["LDS Size"] <= LDS_PER_CU // 2 and u["VGPRs"] + u["AGPRs"] <= 256
+                       for u in few.values()), few
 
 
 def test_one_wavefront_per_simd_kernels_use_the_whole_register_file():
