@@ -113,9 +113,9 @@ int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t t
   if (kv_format == SMLA_KV_F32) return 1;
   // one 4-wave workgroup per CU is resident at a time; each covers 64 (or, for <= 32 heads, 16)
   // heads of one token
-  // (the opt-in fp8 kernel keeps two workgroups per CU, and wants a few more than that so their phases drift apart)
+  // (the opt-in fp8 kernel keeps two workgroups per CU; every further split adds a partial to publish and fold)
   const bool few_fp8 = kv_format == SMLA_KV_FP8_B128 && n_heads <= 32 && few_fp8_enabled();
-  const int slots = few_fp8 ? 4 * device_cus() : device_cus();
+  const int slots = few_fp8 ? 2 * device_cus() : device_cus();
   const int per_wg = n_heads <= 32 ? 16 : 64;
   const long long groups = (long long)n_tokens * ((n_heads + per_wg - 1) / per_wg);
   int want = (int)((slots + groups - 1) / groups);
