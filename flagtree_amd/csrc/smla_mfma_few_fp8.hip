@@ -151,14 +151,11 @@ __global__ __launch_bounds__(kNT, 2) void fwd_few_fp8_kernel(Params p, int n_hbl
   // code free of divergent loads): B operand of S^T, lane = head, k = 32 ks + 8 q4 + j
   bf16x8 qf[kDqk / 32];
   {
+    // (a head past the end reads head 0 again and its results are never stored; nothing touches the
+    // values here, so the compiler waits for Q where the first MFMA uses it, not ahead of the row list)
     const uint16_t* qrow = static_cast<const uint16_t*>(p.q) + ((size_t)t * p.n_heads + (head_ok ? head : 0)) * kDqk + 8 * q4;
-    const uint32_t keep = head_ok ? 0xffffffffu : 0u;
 #pragma unroll
-    for (int ks = 0; ks < kDqk / 32; ++ks) {
-      uint4 raw = *reinterpret_cast<const uint4*>(qrow + 32 * ks);
-      raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
-      qf[ks] = __builtin_bit_cast(bf16x8, raw);
-    }
+    for (int ks = 0; ks < kDqk / 32; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
   }
   if (tid == 0) s_flag = 0;
   translate_entries4(p, seq, rr_first);

@@ -202,17 +202,12 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
   // ---- Q^T fragments: B operand of S^T, lane = head, k = 32*ks + 8*q4 + j
   bf16x8 qf[kDqk / 32];
   {
+    // (every lane loads; a head past the end reads head 0 again and its results are never stored.
+    // Nothing touches the values here: a mask would make the compiler wait for Q ahead of the
+    // row list, which only needs the index values)
     const uint16_t* qrow = static_cast<const uint16_t*>(p.q) + ((size_t)t * p.n_heads + (head_ok ? head : 0)) * kDqk + 8 * q4;
-    // (every lane loads; a head past the end is masked to zero with an AND: conditional loads end
-    // up in branches, and then the compiler waits for all of them wherever an older load -- the
-    // index values -- is first used)
-    const uint32_t keep = head_ok ? 0xffffffffu : 0u;
 #pragma unroll
-    for (int ks = 0; ks < kDqk / 32; ++ks) {
-      uint4 raw = *reinterpret_cast<const uint4*>(qrow + 32 * ks);
-      raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
-      qf[ks] = __builtin_bit_cast(bf16x8, raw);
-    }
+    for (int ks = 0; ks < kDqk / 32; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
   }
   if (tid == 0) s_flag = 0;
   translate_entries(rr_first);               // waits for the index values only; the page lookups overlap the Q loads

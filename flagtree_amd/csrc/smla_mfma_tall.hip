@@ -369,19 +369,12 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
 #pragma unroll
   for (int ht = 0; ht < 2; ++ht) {
     const int hq = head0 + 16 * ht + l16;
-    const bool ok = hq < p.n_heads;
-    // Every lane loads (a head past the end reads head 0 and is masked to zero with an AND, not a
-    // select): conditional loads end up in branches, and loads that "may or may not have been
-    // issued" make the compiler wait for all of them wherever an older load is first used -- here
-    // the index values, which must not wait for Q.
-    const uint16_t* qrow = static_cast<const uint16_t*>(p.q) + ((size_t)t * p.n_heads + (ok ? hq : 0)) * kDqk + 8 * q4;
-    const uint32_t keep = ok ? 0xffffffffu : 0u;
+    // Every lane loads; a head past the end reads head 0 again (its results are never stored).
+    // Nothing touches the values here: whatever consumed them (a mask, say) would make the
+    // compiler wait for Q ahead of the row list, which only needs the index values.
+    const uint16_t* qrow = static_cast<const uint16_t*>(p.q) + ((size_t)t * p.n_heads + (hq < p.n_heads ? hq : 0)) * kDqk + 8 * q4;
 #pragma unroll
-    for (int ks = 0; ks < kDqk / 32; ++ks) {
-      uint4 raw = *reinterpret_cast<const uint4*>(qrow + 32 * ks);
-      raw.x &= keep; raw.y &= keep; raw.z &= keep; raw.w &= keep;
-      qf[ks][ht] = __builtin_bit_cast(bf16x8, raw);
-    }
+    for (int ks = 0; ks < kDqk / 32; ++ks) qf[ks][ht] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
   }
   if (tid == 0) s_redo = 0;
   if (bt_in_lds) {
@@ -520,9 +513,14 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
 
       // ---- prologue: tiles 0 and 1 go out at once, tile 2 rides on the scores of tile 0
       if constexpr (FMT == SMLA_KV_BF16) {
-        hw::wait_vmcnt<0>();   // Q and index loads: the DMA is counted from zero
+        // The moves go out as soon as the row list exists; Q may still be on its way.  Loads
+        // complete in issue order, so waiting for the moves below also waits for everything older.
         for (int it = 0; it < min(n_tiles, 2); ++it) fetch_whole(it);
         wait_dma(n_tiles > 1 ? 1 : 0);
+        // Tell the compiler that Q has arrived (it cannot see the wait above): otherwise it would
+        // wait for Q inside the first tile's MFMA stream, and with it for the moves issued there.
+#pragma unroll
+        for (int ks = 0; ks < kDqk / 32; ++ks) hw::wait_for_loads_of(qf[ks][0], qf[ks][1]);
       } else {
         for (int it = 0; it < min(n_tiles, kSlots - 1); ++it) fetch_whole(it);
       }
