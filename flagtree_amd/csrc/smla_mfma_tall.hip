@@ -671,7 +671,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   __syncthreads();                                                 // staged blocks and scalar exchange are done
   if (g == 0) s_x[wave][c32] = inv;                                // per-row normaliser
   hw::wave_lds_order();
-  const int n_rows = min(32, p.n_heads - head0);                   // head rows that exist (wave-uniform)
+  const int n_rows = max(0, min(32, p.n_heads - head0));           // head rows that exist (wave-uniform; 0: the whole head group lies past the last head)
   const int col4 = kDvHalf * dh + 4 * lane;                        // this lane's 4 dv columns
   auto staged = [&](int row) { return *reinterpret_cast<const float4*>(stage + row * kStageStride + 4 * lane); };
   auto store_bf16x4 = [&](int row, float4 v) {
@@ -773,11 +773,14 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
           const float4 a4 = staged(r0 + j);
           v[j] = f32x4{a4.x, a4.y, a4.z, a4.w};
         }
-      } else {
+      } else if (n_rows > 0) {
         const hw::buffer_rsrc src = hw::make_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0) * kDv);
 #pragma unroll
         for (int j = 0; j < 16; ++j)
           v[j] = hw::load_b128_agent(src, (uint32_t)((min(r0 + j, n_rows - 1) * kDv + col4) * 4));
+      } else {                                 // a head group without heads has no partials to read (and stores nothing)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
 #pragma unroll
       for (int j = 0; j < 16; ++j) {

@@ -49,7 +49,7 @@ def build(verbose=False, force=False):
         if verbose and out.strip():
             print(out)
     if procs or not os.path.exists(LIB_PATH):
-        res = subprocess.run([CXX, "-shared", "-o", LIB_PATH] + objs, stdout=subprocess.PIPE,
+        res = subprocess.run([CXX, "-shared", "-rdynamic", "-o", LIB_PATH] + objs, stdout=subprocess.PIPE,
                              stderr=subprocess.STDOUT, text=True)
         if res.returncode != 0:
             raise RuntimeError("emulator link failed:\n" + res.stdout[-4000:])

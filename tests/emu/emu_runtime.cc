@@ -1,11 +1,14 @@
 // Fiber scheduler, rendezvous, LDS arena and deferred global -> LDS moves of the CPU emulator.
 #include "emu_runtime.h"
 
+#include <execinfo.h>
+#include <signal.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 #include <sys/mman.h>
+#include <unistd.h>
 
 #include <algorithm>
 #include <random>
@@ -276,8 +279,43 @@ void dma_wait(int allowed_in_flight) {
   q.erase(q.begin(), q.begin() + land);
 }
 
+namespace {
+// A stray global access by an emulated kernel: say where it happened before the process dies.
+void on_segv(int sig, siginfo_t* info, void*) {
+  char buf[256];
+  const int n = snprintf(buf, sizeof(buf),
+                         "[emu] signal %d at address %p in block (%u,%u,%u), thread %d of the workgroup\n", sig,
+                         info ? info->si_addr : nullptr, g_block_idx.x, g_block_idx.y, g_block_idx.z,
+                         g_cur ? g_cur->lane.flat : -1);
+  if (n > 0) (void)!write(2, buf, (size_t)n);
+  void* frames[32];
+  const int depth = backtrace(frames, 32);
+  backtrace_symbols_fd(frames, depth, 2);
+  signal(sig, SIG_DFL);
+  raise(sig);
+}
+void install_handler() {
+  static bool done = false;
+  if (done) return;
+  done = true;
+  static char alt[1 << 16];
+  stack_t ss;
+  ss.ss_sp = alt;
+  ss.ss_size = sizeof(alt);
+  ss.ss_flags = 0;
+  sigaltstack(&ss, nullptr);
+  struct sigaction sa;
+  memset(&sa, 0, sizeof(sa));
+  sa.sa_sigaction = on_segv;
+  sa.sa_flags = SA_SIGINFO | SA_ONSTACK | SA_RESETHAND;
+  sigaction(SIGSEGV, &sa, nullptr);
+  sigaction(SIGBUS, &sa, nullptr);
+}
+}  // namespace
+
 void launch(Dim3 grid, Dim3 block, const std::function<void()>& body) {
   if (g_cur != nullptr) fail("launch from inside a kernel");
+  install_handler();
   g_launches++;
   g_block_dim = block;
   g_grid_dim = grid;
