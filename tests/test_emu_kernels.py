@@ -106,6 +106,74 @@ def test_fp8_records(heads, n_splits):
 
 
 @pytest.fixture
+def wide_kernel(monkeypatch):
+    """Routes many-heads bf16 launches to the 128-heads-per-workgroup kernel (opt-in until it is measured)."""
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")
+
+
+@pytest.mark.parametrize("heads,n_splits,topk", [(128, 1, 300), (128, 2, 300), (64, 3, 200), (96, 1, 100), (40, 2, 70),
+                                                 (200, 2, 130), (128, 4, 1100), (65, 3, 200), (129, 2, 90)])
+def test_128_heads_per_workgroup_kernel(wide_kernel, heads, n_splits, topk):
+    from flagtree_amd import workloads
+    cfg = workloads.decode_bf16("cpu", batch=2, heads=heads, pages_per_seq=20, topk=topk, pad_frac=0.07)
+    out, lse = _forward_all_ways(cfg, n_splits)
+    _check(cfg, out, lse)
+    os.environ.pop("FLAGTREE_SMLA_WIDE")
+    out1, lse1, rc = harness.forward(cfg, n_splits=n_splits)             # the first kernel: same results to the bar, not to the bit
+    assert rc == 0 and not torch.equal(out1.view(torch.int16), out.view(torch.int16))
+    assert max_abs(to_np(out1), to_np(out)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse)) <= 1e-5
+
+
+def test_128_heads_kernel_edge_cases_redo_prefill_and_dense(wide_kernel):
+    from flagtree_amd import workloads
+    g = torch.Generator().manual_seed(7)
+    kv = (torch.randn((300, 576), generator=g) * 0.1).to(torch.bfloat16)
+    q = (torch.randn((6, 128, 576), generator=g) * 0.1).to(torch.bfloat16)
+    idx = torch.full((6, 70), -1, dtype=torch.int32)
+    idx[1, 33] = 5
+    idx[2, :] = torch.randperm(300, generator=g)[:70].to(torch.int32)
+    idx[3, :35] = 17
+    idx[4, ::2] = torch.arange(35, dtype=torch.int32)
+    idx[5, 0] = 299
+    idx[5, 1] = 300
+    cfg = dict(q=q, kv_cache=kv, indices=idx, block_table=None, page_size=64, sm_scale=576 ** -0.5, kv_format="bf16")
+    for ns in (1, 2):
+        out, lse = _forward_all_ways(cfg, ns)
+        _check(cfg, out, lse)
+        o, l = to_np(out), to_np(lse)
+        assert (o[0] == 0).all() and np.isneginf(l[0]).all()
+        assert np.array_equal(o[1], np.broadcast_to(to_np(kv)[5, :512], (128, 512)))
+    # the exact two-pass path
+    kv = (torch.randn((400, 576), generator=g) * 4.0).to(torch.bfloat16)
+    kv[:64] *= 0.01
+    q = (torch.randn((2, 128, 576), generator=g) * 4.0).to(torch.bfloat16)
+    cfg = dict(q=q, kv_cache=kv, indices=torch.arange(200, dtype=torch.int32).repeat(2, 1), block_table=None, page_size=64,
+               sm_scale=576 ** -0.5, kv_format="bf16")
+    ro, rl = run_oracle(cfg)
+    for ns in (1, 2):
+        out, lse = _forward_all_ways(cfg, ns)
+        assert max_abs(to_np(lse), rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
+        assert max_abs(to_np(out), ro) <= 1.2e-2 * max(1.0, float(np.abs(ro).max()))
+    # causal prefill, lists longer than a chunk, dense decode with a cap
+    cfg = workloads.prefill_causal_bf16("cpu", tokens=40, heads=128, topk=48)
+    out, lse = _forward_all_ways(cfg, 1)
+    _check(cfg, out, lse)
+    cfg = workloads.decode_bf16("cpu", batch=1, heads=128, pages_per_seq=40, topk=2100, pad_frac=0.05)
+    out, lse = _forward_all_ways(cfg, 1)
+    _check(cfg, out, lse)
+    cfg = workloads.decode_bf16("cpu", batch=3, heads=128, pages_per_seq=5, topk=64, pad_frac=0.0)
+    lens = torch.tensor([300, 1, 129], dtype=torch.int32)
+    didx = torch.full((3, 1, 320), -1, dtype=torch.int32)
+    for b, n in enumerate(lens.tolist()):
+        didx[b, 0, :n] = torch.arange(n, dtype=torch.int32)
+    qn, kv_small, phys_small, _ = oracle_inputs(dict(cfg, indices=didx))
+    for cap in (0.0, 0.02):
+        wo, wl = oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfg["sm_scale"], 512, logit_cap=cap)
+        out, lse = _forward_all_ways(cfg, 2, dense_lens=lens, logit_cap=cap)
+        assert max_abs(to_np(lse), wl) <= 1e-3 and max_abs(to_np(out), wo) <= 1e-2
+
+
+@pytest.fixture
 def few_fp8_kernel(monkeypatch):
     """Routes few-heads fp8 launches to the two-workgroups-per-CU kernel (opt-in until it is measured)."""
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
@@ -287,7 +355,7 @@ def test_dense_decode_with_logit_cap(heads, fmt, std, cap, min_diff):
 
 
 @pytest.mark.parametrize("seed", list(range(12)))
-@pytest.mark.parametrize("few_fp8", [False, True])
+@pytest.mark.parametrize("few_fp8", [False, True, "wide"])
 def test_random_shapes_against_oracle(seed, few_fp8, monkeypatch):
     """Seeded draws over head counts, list lengths, page sizes, tokens per sequence, split counts,
     padding patterns, page tables with holes and both cache formats (the GPU suite's recipe at sizes
@@ -303,7 +371,11 @@ def test_random_shapes_against_oracle(seed, few_fp8, monkeypatch):
     n_splits = [1, 2, 3, 5][int(rng.integers(4))]
     paged = rng.random() < 0.7
     ctx = int(rng.choice([64, 300, 1200]))
-    if few_fp8:
+    if few_fp8 == "wide":
+        if fmt != "bf16" or heads <= 32:
+            pytest.skip("the opt-in kernel covers many heads over a bf16 cache")
+        monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")
+    elif few_fp8:
         if fmt != "fp8_e4m3_b128" or heads > 32:
             pytest.skip("the opt-in kernel covers few heads over an fp8 cache")
         monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")

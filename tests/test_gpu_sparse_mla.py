@@ -734,3 +734,58 @@ def test_column_split_fp8_kernel_edge_cases_and_dense(dev, few_fp8_kernel):
     qn, kv_small, phys_small, _ = oracle_inputs(cfgd)
     wo, wl = oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfgd["sm_scale"], 512, logit_cap=cap)
     assert max_abs(to_np(lse), wl.reshape(B, 16)) <= 1e-3 and max_abs(to_np(o), wo.reshape(B, 16, 512)) <= 1e-2
+
+
+# ---- the 128-heads-per-workgroup bf16 kernel (opt-in until it has been measured) ----------------
+
+@pytest.fixture
+def wide_kernel(monkeypatch):
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")
+
+
+@pytest.mark.parametrize("heads,n_splits,topk", [(128, 1, 512), (128, 2, 512), (64, 3, 300), (200, 2, 700), (128, None, 2048),
+                                                 (65, 3, 200)])
+def test_128_heads_kernel_against_oracle(dev, wide_kernel, heads, n_splits, topk):
+    from flagtree_amd import workloads
+    cfg = workloads.decode_bf16(dev, batch=5, heads=heads, pages_per_seq=40, topk=topk, pad_frac=0.03)
+    out, lse = _fwd(cfg, n_splits=n_splits)
+    _check(cfg, out, lse)
+
+
+def test_128_heads_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch):
+    """Headline decode size: the two kernels agree to the bar (they sum in different orders), and a
+    slice of the batch agrees with the oracle."""
+    from flagtree_amd import workloads
+    cfg = workloads.decode_bf16(dev)
+    out0, lse0 = _fwd(cfg)
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")
+    out1, lse1 = _fwd(cfg)
+    torch.cuda.synchronize()
+    assert not torch.equal(out0, out1)                       # it really is the other kernel
+    assert max_abs(to_np(out1), to_np(out0)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse0)) <= 1e-4
+    sub = dict(cfg, q=cfg["q"][:2], indices=cfg["indices"][:2], block_table=cfg["block_table"][:2])
+    ro, rl = run_oracle(sub)
+    H = cfg["q"].shape[-2]
+    assert max_abs(to_np(out1[:2]).reshape(2, H, 512), ro) <= OUT_TOL and max_abs(to_np(lse1[:2]).reshape(2, H), rl) <= LSE_TOL
+
+
+def test_128_heads_kernel_prefill_and_redo(dev, wide_kernel):
+    from flagtree_amd import workloads
+    cfg = workloads.prefill_causal_bf16(dev, tokens=300, heads=128, topk=256)
+    out, lse = _fwd(cfg)
+    rows = slice(130, 170)                                   # lists of 131..170 entries: more than one chunk of 128
+    sub = dict(cfg, q=cfg["q"][:, rows], indices=cfg["indices"][:, rows])
+    ro, rl = run_oracle(sub)
+    assert max_abs(to_np(out[:, rows]).reshape(ro.shape), ro) <= OUT_TOL
+    assert max_abs(to_np(lse[:, rows]).reshape(rl.shape), rl) <= LSE_TOL
+    g = torch.Generator().manual_seed(3)
+    kv = (torch.randn((400, 576), generator=g) * 4.0).to(torch.bfloat16)
+    kv[:64] *= 0.01
+    q = (torch.randn((2, 128, 576), generator=g) * 4.0).to(torch.bfloat16)
+    cfg = dict(q=q.to(dev), kv_cache=kv.to(dev), indices=torch.arange(200, dtype=torch.int32).repeat(2, 1).to(dev),
+               block_table=None, page_size=64, sm_scale=576 ** -0.5, kv_format="bf16")
+    ro, rl = run_oracle(cfg)
+    for ns in (1, 2):
+        out, lse = _fwd(cfg, n_splits=ns)
+        assert max_abs(to_np(lse).reshape(rl.shape), rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
+        assert max_abs(to_np(out).reshape(ro.shape), ro) <= 1.2e-2 * max(1.0, float(np.abs(ro).max()))
