@@ -37,6 +37,10 @@ __device__ __forceinline__ bf16x4 lds_read_tr16_b64(const void* shared_object) {
   return __builtin_bit_cast(bf16x4, v);
 }
 
+// This lane's position in its wavefront, from the hardware's lane counter (two instructions; a
+// value the compiler does not connect with threadIdx, so it is recomputed where it is used).
+__device__ __forceinline__ int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
 // Marks a point where lanes of ONE wavefront hand data to each other through LDS (one lane
 // writes, another reads, no workgroup barrier in between).  Nothing is needed on the hardware: a
 // wavefront's lanes execute an instruction together and its LDS accesses complete in program
@@ -52,6 +56,17 @@ __device__ __forceinline__ void wave_lds_order() {}
 // serialise them against LDS reads of other ring slots.
 __device__ __forceinline__ void dma_b128(const void* lane_src, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(lane_src), "s"(lds_base) : "memory", "m0");
+}
+// A move in which only lanes 0 .. N-1 take part (the others' LDS pieces stay as they are).  The
+// execution mask is narrowed and restored around the instruction right here, so that no branch
+// cuts the surrounding instruction stream in two; the move counts once for vmcnt like any other.
+// Every lane of the wavefront must be active at the call.
+template <int N>
+__device__ __forceinline__ void dma_b128_first_lanes(const void* lane_src, uint32_t lds_base) {
+  static_assert(N > 0 && N < 32, "the mask is written as a 32-bit literal");
+  uint64_t saved;
+  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %3\n\ts_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b64 exec, %0"
+               : "=&s"(saved) : "v"(lane_src), "s"(lds_base), "n"((1u << N) - 1u) : "memory", "m0");
 }
 // scalar base + per-lane byte offset
 __device__ __forceinline__ void dma_b128(uint32_t lane_off, uint64_t wave_base, uint32_t lds_base) {
@@ -79,6 +94,9 @@ template <typename... T>
 __device__ __forceinline__ void wait_for_loads_of(const T&... v) { (..., [](const auto& x) { asm volatile("" ::"v"(x)); }(v)); }
 template <typename... T>
 __device__ __forceinline__ void pin(T&... v) { (..., [](auto& x) { asm volatile("" : "+v"(x)); }(v)); }
+// the same for a wave-uniform value (it stays in a scalar register).  Also the way to keep what
+// is derived from the value from being computed once, far ahead, and held in registers since.
+__device__ __forceinline__ void pin_uniform(uint32_t& v) { asm volatile("" : "+s"(v)); }
 
 // mask = 2 * mask + (x > y) / (x == y), unsigned: a compare into vcc and an add with carry-in, two
 // vector instructions a bit (the compiler's own lowering takes three and a half); the wait state

@@ -13,6 +13,8 @@
 //   3. accumulates output columns 256*dh .. +255 over all 32 tokens of tile i
 //        O[32 heads x 256] += P[32 heads x 32 tok] . V[32 tok x 256]    v_mfma_f32_32x32x16_bf16
 //        (A = P from LDS, B = V through transposing LDS reads of the same tile).
+// An fp8 cache takes the same road with one more stage: raw records -> LDS by the same moves,
+// LDS -> LDS conversion to bf16 tiles under the P.V MFMAs one tile ahead of the scores (Fp8Pipe).
 // The workgroups of one token (head blocks x splits) are given ids 8 apart so they land on the
 // same XCD: the head blocks share the L2 for the rows they both gather, and the splits are
 // merged by whichever workgroup of a (token, head block) finishes last.
@@ -112,61 +114,95 @@ struct DmaTile {
   }
 };
 
-__device__ __forceinline__ uint32_t rope_slot(int r, int c) {     // byte offset of RoPE chunk c of tile row r
+__device__ __forceinline__ uint32_t rope_slot(int r, int c) {     // byte offset of RoPE chunk c of tile row r in a tile's RoPE block
   const int p = r >> 1;
-  return kRopeBase + p * 256 + ((((r & 1) << 3) | (c ^ (p & 7))) << 4);
+  return p * 256 + ((((r & 1) << 3) | (c ^ (p & 7))) << 4);
 }
 
-// fp8 records are dequantised in registers on their way to LDS: chunk col 0..31 = 16 e4m3
-// values (block scale col/8), col 32 = the 4 scales, col 33..40 = 8 bf16 rope values;
-// LDS gets bf16(float(e4m3) * scale).  One call moves a whole 32-row tile, synchronously, two chunks per
-// thread at a time.
-struct Fp8Stager {
-  static constexpr int kChunksPerRow = kRowBytesFp8 / 16;    // 41
-  static constexpr int kIters = (kTN * kChunksPerRow + kNT - 1) / kNT;   // 6
-  static constexpr int kBatch = 2;             // chunks a thread holds at a time: the kernel has few registers to spare
-  // moves chunks tid + kNT * (i0 .. i0 + kBatch - 1) of the tile
-  __device__ __forceinline__ void move(const uint8_t* kv, const int32_t* rows, int e0, int n_valid, uint8_t* tile, int tid, int i0) {
-    uint4 v[kBatch];
-    float sc[kBatch];
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      const int c = tid + kNT * (i0 + i);
-      if (c < kTN * kChunksPerRow) {
-        const int row = c / kChunksPerRow, col = c % kChunksPerRow;
-        const int e = min(e0 + row, n_valid - 1);
-        const uint8_t* rec = kv + (size_t)rows[e] * kRowBytesFp8;
-        v[i] = *reinterpret_cast<const uint4*>(rec + col * 16);
-        sc[i] = col < 32 ? *reinterpret_cast<const float*>(rec + kFp8ScaleOff + 4 * (col >> 3)) : 0.f;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      const int c = tid + kNT * (i0 + i);
-      const int row = c / kChunksPerRow, col = c % kChunksPerRow;
-      uint8_t* dst = tile + row * kMainStride;
-      const int sw = swz(row);
-      if (c >= kTN * kChunksPerRow) {
-      } else if (col < 32) {
-        const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
-        uint32_t o[8];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[k], false);
-          const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[k], true);
-          o[2 * k] = pack_bf16(lo[0] * sc[i], lo[1] * sc[i]);
-          o[2 * k + 1] = pack_bf16(hi[0] * sc[i], hi[1] * sc[i]);
-        }
-        *reinterpret_cast<uint4*>(dst + (((2 * col) ^ sw) << 4)) = make_uint4(o[0], o[1], o[2], o[3]);
-        *reinterpret_cast<uint4*>(dst + (((2 * col + 1) ^ sw) << 4)) = make_uint4(o[4], o[5], o[6], o[7]);
-      } else if (col > 32) {
-        *reinterpret_cast<uint4*>(tile + rope_slot(row, col - 33)) = v[i];
-      }
+// fp8 records (512 e4m3 values, 4 float scales, 64 bf16 RoPE values = 656 bytes) reach LDS raw,
+// by the same global -> LDS moves, and are dequantised from LDS to LDS: no register waits for
+// memory.  Wavefront w owns tile rows 8w .. 8w+7 from end to end.  Move j = 0..3 fetches the value
+// chunks of its rows 2j and 2j+1 (lane l: row 2j + l/32, chunk l%32) into 1 KB of its raw block,
+// move 4 the eight scale chunks (lanes 0..7, one row each) into the 128 bytes behind them, move 5
+// the RoPE parts straight into the tile's RoPE block (they are bf16 already).  Later every lane
+// turns the four value chunks it fetched itself (raw block byte 16*l + 1024*k) into
+// bf16(float(e4m3) * scale) in the tile body.  Only the wavefront's own moves feed its
+// conversion, so a wait on its own counter is all the synchronisation the raw data needs, and a
+// raw block can be refilled as soon as it is converted.
+// LDS: three tile bodies (one being multiplied, one being scored, one being written), three RoPE
+// blocks (scored, landed, in flight) and two raw blocks per wavefront (converting, in flight).
+struct Fp8Pipe {
+  static constexpr int kRawWave = 8 * (kFp8ScaleOff + 16);     // 4224 bytes: a wavefront's 8 rows, values then scales
+  static constexpr int kRawScales = 8 * kFp8ScaleOff;          // 4096: where the scale chunks start
+  static constexpr int kRawSlot = 4 * kRawWave;                // 16896
+  static constexpr int kSteps = 6;                             // move instructions per wavefront per tile
+  static constexpr int kBodies = 3, kRopes = 3, kRaws = 2;
+  static constexpr int kRopeRing = kBodies * kRopeBase;        // byte offsets in the ring area
+  static constexpr int kRawRing = kRopeRing + kRopes * (kTN * 128);
+  static constexpr int kRingBytes = kRawRing + kRaws * kRawSlot;      // 144384
+  const uint8_t* kv;
+  uint32_t raw_lds, rope_lds;
+  int32_t rid;
+  int wave, lane;
+  // raw_lds_: this wavefront's raw block, rope_lds_: the tile's RoPE block
+  __device__ __forceinline__ void begin(const uint8_t* kv_, const int32_t* rows, int e0, int n_valid,
+                                        uint32_t raw_lds_, uint32_t rope_lds_, int wave_, int lane_) {
+    kv = kv_; raw_lds = raw_lds_; rope_lds = rope_lds_; wave = wave_; lane = lane_;
+    rid = rows[min(e0 + (lane & 31), n_valid - 1)];               // lane l holds the row id of tile row l % 32
+  }
+  __device__ __forceinline__ void step(int j) const {
+    if (j < 4) {
+      const int32_t trow = __shfl(rid, 8 * wave + 2 * j + (lane >> 5));
+      hw::dma_b128(kv + (size_t)trow * kRowBytesFp8 + (lane & 31) * 16, raw_lds + 1024 * j);
+    } else if (j == 4) {
+      const int32_t trow = __shfl(rid, 8 * wave + (lane & 7));
+      hw::dma_b128_first_lanes<8>(kv + (size_t)trow * kRowBytesFp8 + kFp8ScaleOff, raw_lds + kRawScales);
+    } else {
+      const int pair = 4 * wave + (lane >> 4);
+      const int r = 2 * pair + ((lane >> 3) & 1), c = (lane & 7) ^ (pair & 7);
+      const int32_t trow = __shfl(rid, r);
+      hw::dma_b128(kv + (size_t)trow * kRowBytesFp8 + kFp8ScaleOff + 16 + c * 16, rope_lds + wave * 1024);
     }
   }
-  __device__ __forceinline__ void move_tile(const uint8_t* kv, const int32_t* rows, int e0, int n_valid, uint8_t* tile, int tid) {
+};
+
+// The conversion of one tile is 4 chunks of 16 values per lane: chunk k is column chunk l % 32 of
+// the wavefront's row l/32 + 2k.  load / half / store are separate so that a caller can thread
+// them through an MFMA stream.
+struct Fp8Convert {
+  uint4 v;
+  float sc;
+  uint32_t o[8];
+  const uint8_t* raw;      // this wavefront's raw block
+  uint8_t* body;           // the tile body being written
+  int wave, lane;
+  __device__ __forceinline__ void load(int k) {
+    v = *reinterpret_cast<const uint4*>(raw + 16 * lane + 1024 * k);
+    sc = *reinterpret_cast<const float*>(raw + Fp8Pipe::kRawScales + 16 * (lane >> 5) + 4 * ((lane & 31) >> 3) + 32 * k);
+  }
+  __device__ __forceinline__ void half(int h) {
+    const uint32_t w[2] = {h == 0 ? v.x : v.z, h == 0 ? v.y : v.w};
 #pragma unroll
-    for (int i0 = 0; i0 < kIters; i0 += kBatch) move(kv, rows, e0, n_valid, tile, tid, i0);
+    for (int k = 0; k < 2; ++k) {
+      const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[k], false);
+      const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[k], true);
+      o[4 * h + 2 * k] = pack_bf16(lo[0] * sc, lo[1] * sc);
+      o[4 * h + 2 * k + 1] = pack_bf16(hi[0] * sc, hi[1] * sc);
+    }
+  }
+  __device__ __forceinline__ void store(int k) {
+    // tile row 8*wave + l/32 + 2k, chunks 2*col and 2*col + 1.  With row0 the row of k = 0:
+    // swz(row) = swz(row0) ^ (8 * (k & 1) | (k >> 1)), so one per-lane offset serves all four chunks.
+    const int row0 = 8 * wave + (lane >> 5), col = lane & 31;
+    int off = row0 * kMainStride + (((2 * col) ^ swz(row0)) << 4);
+    hw::pin(off);                                                  // (worked out here, not kept in four registers from the top of the kernel)
+    off = (off ^ (((8 * (k & 1)) | (k >> 1)) << 4)) + 2 * k * kMainStride;
+    *reinterpret_cast<uint4*>(body + off) = make_uint4(o[0], o[1], o[2], o[3]);
+    *reinterpret_cast<uint4*>(body + (off ^ 16)) = make_uint4(o[4], o[5], o[6], o[7]);
+  }
+  __device__ __forceinline__ void whole_tile() {     // (one chunk at a time: where this is called, registers are scarce)
+#pragma unroll 1
+    for (int k = 0; k < 4; ++k) { load(k); half(0); half(1); store(k); }
   }
 };
 
@@ -187,13 +223,13 @@ enum { kPassFast = 0, kPassMax = 1, kPassFinal = 2 };
 constexpr int kPrefetchA = 5;                 // K fragments ahead in the score loop
 constexpr int kPrefetchB = 6;                 // V fragments ahead in the P.V loop
 
-// S^T = K_rows . Q^T : tile rows tok0 .. tok0+15 against this wavefront's 32 heads (two head
+// S^T = K_rows . Q^T : tile rows tok0 .. tok0+15 (body at `tile`, RoPE block at `rope`) against this wavefront's 32 heads (two head
 // tiles of 16: heads 0..15 and 16..31 of the group).  Four independent accumulation chains
 // (head tile x parity of the k-step) keep dependent MFMAs apart; sa[2*ht] + sa[2*ht+1] is the
 // score block of head tile ht.  `side(ks)` is called once per k-step: the caller threads DMA
 // issue through the MFMA stream.
 template <typename Side>
-__device__ __forceinline__ void tile_scores(uint32_t tile, int tok0, const bf16x8 (&qf)[kDqk / 32][2],
+__device__ __forceinline__ void tile_scores(uint32_t tile, uint32_t rope, int tok0, const bf16x8 (&qf)[kDqk / 32][2],
                                             f32x4 (&sa)[4], int lane, Side side) {
   constexpr int kSteps = kDqk / 32, kMainSteps = kDv / 32;     // 18 k-steps of 32, 16 of them in the NoPE part
   const int t = tok0 + (lane & 15), q4 = lane >> 4;
@@ -202,7 +238,7 @@ __device__ __forceinline__ void tile_scores(uint32_t tile, int tok0, const bf16x
   const uint32_t kmain = tile + t * kMainStride + ((q4 ^ swz(t)) << 4);
   auto frag = [&](int ks) {
     if (ks < kMainSteps) return lds_read_b128((kmain ^ (uint32_t)((ks & 3) << 6)) + (ks >> 2) * 256);
-    return lds_read_b128(tile + rope_slot(t, 4 * (ks - kMainSteps) + q4));
+    return lds_read_b128(rope + rope_slot(t, 4 * (ks - kMainSteps) + q4));
   };
 #pragma unroll
   for (int i = 0; i < 4; ++i) sa[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -234,8 +270,8 @@ __device__ __forceinline__ void tile_scores(uint32_t tile, int tok0, const bf16x
 // `valu(i)` is independent vector-ALU work of the caller (a slice of the softmax of the next tile).
 // With kPinValu it is pinned between MFMA i and MFMA i+1 by scheduling barriers, so it issues
 // while the matrix core is busy with MFMA i; the LDS reads then simply stay in source order
-// (they are written kPrefetchB steps ahead of their use).
-template <bool kPinValu, typename Side, typename Valu>
+// (they are written kAhead steps ahead of their use).
+template <bool kPinValu, int kAhead = kPrefetchB, typename Side, typename Valu>
 __device__ __forceinline__ void tile_accumulate(uint32_t tile, uint32_t pbuf, int dv0, f32x16 (&acc)[kAccTiles],
                                                 int lane, Side side, Valu valu) {
   constexpr int kSteps = 2 * kAccTiles;
@@ -259,10 +295,10 @@ __device__ __forceinline__ void tile_accumulate(uint32_t tile, uint32_t pbuf, in
     hi[i] = lds_read_tr((vbase ^ (uint32_t)(64 * dt + 16)) + (16 * s2 + 4) * kMainStride);
   };
 #pragma unroll
-  for (int i = 0; i < kPrefetchB; ++i) load(i);
+  for (int i = 0; i < kAhead; ++i) load(i);
 #pragma unroll
   for (int i = 0; i < kSteps; ++i) {
-    if (i + kPrefetchB < kSteps) load(i + kPrefetchB);
+    if (i + kAhead < kSteps) load(i + kAhead);
     const bf16x8 bv = __builtin_shufflevector(lo[i], hi[i], 0, 1, 2, 3, 4, 5, 6, 7);
     acc[i % kAccTiles] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa[i / kAccTiles], bv, acc[i % kAccTiles], 0, 0, 0);
     side(i);
@@ -275,10 +311,10 @@ __device__ __forceinline__ void tile_accumulate(uint32_t tile, uint32_t pbuf, in
   if constexpr (!kPinValu) {
     __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
-    for (int i = 0; i < kPrefetchB; ++i) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    for (int i = 0; i < kAhead; ++i) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
     for (int i = 0; i < kSteps; ++i) {
-      if (i + kPrefetchB < kSteps) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      if (i + kAhead < kSteps) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
   }
@@ -294,7 +330,10 @@ __device__ __forceinline__ void wait_dma(int younger_tiles) {
 
 template <int FMT, bool CAP>
 __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) {
-  __shared__ __attribute__((aligned(1024))) uint8_t s_tile[kSlots][kTileBytes];   // swizzle xors need 1 KB alignment
+  // the ring area: bf16 has four whole tiles (body + RoPE block each); fp8 see Fp8Pipe
+  constexpr bool kFp8 = FMT == SMLA_KV_FP8_B128;
+  constexpr int kRingBytes = kFp8 ? Fp8Pipe::kRingBytes : kSlots * kTileBytes;
+  __shared__ __attribute__((aligned(1024))) uint8_t s_ring[kRingBytes];           // swizzle xors need 1 KB alignment
   __shared__ __attribute__((aligned(16))) uint8_t s_p[2][2][kPBytes];             // [tile parity][head group]
   __shared__ int32_t s_rows[kChunk];
   __shared__ float s_x[4][32];                                    // per-head scalars exchanged inside a pair
@@ -302,7 +341,6 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   __shared__ int s_nvalid;
   __shared__ int s_cnt[4];
   __shared__ int s_redo;
-  [[maybe_unused]] __shared__ __attribute__((aligned(16))) uint32_t s_sink[64];   // where the fp8 path's L2 warm-up loads land
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -341,7 +379,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     }
   };
   auto translate_entries = [&](int32_t (&rr)[4]) { translate_entries4(p, seq, rr); };
-  // ---- this sequence's page-table row goes global -> LDS (into ring slot 3, which stays free
+  // ---- this sequence's page-table row goes global -> LDS (into the last tile body, which stays free
   // until the first chunk's row list exists) while the indices and Q are on their way, so the
   // first chunk's translation reads LDS instead of paying a second dependent trip to memory.
   // It is issued ahead of the index loads: memory operations complete in order, so once a
@@ -350,7 +388,8 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   const int32_t* bt_row = p.block_table ? p.block_table + (size_t)seq * p.bt_stride : nullptr;
   const bool bt_in_lds = bt_row != nullptr && p.bt_stride <= kBtLdsMax && (p.bt_stride & 3) == 0 &&
                          ((uintptr_t)bt_row & 15) == 0;
-  const uint32_t lds_bt = hw::lds_addr(&s_tile[kSlots - 1][0]);
+  uint8_t* const bt_stage = &s_ring[kFp8 ? (Fp8Pipe::kBodies - 1) * kRopeBase : (kSlots - 1) * kTileBytes];
+  const uint32_t lds_bt = hw::lds_addr(bt_stage);
   if (bt_in_lds) {
     for (int c = wave; 256 * c < p.bt_stride; c += 4) {            // 1 KB (256 entries) per instruction
       const int e = 256 * c + 4 * lane;
@@ -382,7 +421,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     // issued behind them stay in flight); the page-table DMA is older, so it is complete as well.
     hw::wait_for_loads_of(rr_first[0], rr_first[1], rr_first[2], rr_first[3]);
     __syncthreads();
-    const int32_t* bt_s = reinterpret_cast<const int32_t*>(&s_tile[kSlots - 1][0]);
+    const int32_t* bt_s = reinterpret_cast<const int32_t*>(bt_stage);
 #pragma unroll
     for (int k = 0; k < 4; ++k) rr_first[k] = translate_index(p, rr_first[k], bt_s);
   } else {
@@ -401,7 +440,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // already is in base-2 units
   const float sc2 = CAP ? 1.f : p.sm_scale * kLog2e;
   [[maybe_unused]] const LogitCap cap(p.sm_scale, CAP ? p.logit_cap : 1.f);
-  const uint32_t lds_tile = hw::lds_addr(&s_tile[0][0]);
+  const uint32_t lds_tile = hw::lds_addr(&s_ring[0]);
   const uint32_t lds_p = hw::lds_addr(&s_p[0][0][0]);
   const int partner = wave ^ 1;
 
@@ -449,17 +488,42 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
       const int n_tiles = (n_valid + kTN - 1) / kTN;
       if (n_tiles == 0) continue;
 
-      // ---- tile movers.  Tile `it` lives in ring slot it % kSlots.
-      [[maybe_unused]] Fp8Stager stg;
+      // ---- tile movers.  bf16: tile `it` lives in ring slot it % kSlots.  fp8: its body in
+      // body it % 3, its RoPE block in block it % 3, its raw records in raw block it % 2.
+      [[maybe_unused]] Fp8Pipe pipe;
+      [[maybe_unused]] Fp8Convert cv;
       DmaTile dma;
-      auto tile_addr = [&](int it) { return lds_tile + (it & (kSlots - 1)) * kTileBytes; };
-      auto fetch_whole = [&](int it) {       // all of a tile at once (prologue)
-        if constexpr (FMT == SMLA_KV_BF16) {
+      // (fp8: the ring's address is taken afresh for every chunk, so that the per-lane addresses
+      // of the first tiles are worked out here rather than once at the top of the kernel and
+      // then kept in registers, which that variant does not have to spare)
+      uint32_t ring = lds_tile;
+      if constexpr (kFp8) hw::pin_uniform(ring);
+      auto tile_addr = [&](int it) {
+        if constexpr (kFp8) return ring + (uint32_t)(it % Fp8Pipe::kBodies) * kRopeBase;
+        else return ring + (it & (kSlots - 1)) * kTileBytes;
+      };
+      auto rope_addr = [&](int it) {
+        if constexpr (kFp8) return ring + Fp8Pipe::kRopeRing + (uint32_t)(it % Fp8Pipe::kRopes) * (kTN * 128);
+        else return ring + (it & (kSlots - 1)) * kTileBytes + kRopeBase;
+      };
+      [[maybe_unused]] auto pipe_begin = [&](int it) {
+        pipe.begin(kv, s_rows, it * kTN, n_valid,
+                   ring + Fp8Pipe::kRawRing + (it & 1) * Fp8Pipe::kRawSlot + wave * Fp8Pipe::kRawWave, rope_addr(it), wave, lane);
+      };
+      [[maybe_unused]] auto convert_begin = [&](int it) {
+        cv.raw = &s_ring[Fp8Pipe::kRawRing + (it & 1) * Fp8Pipe::kRawSlot + wave * Fp8Pipe::kRawWave];
+        cv.body = &s_ring[(it % Fp8Pipe::kBodies) * kRopeBase];
+        cv.wave = wave; cv.lane = lane;
+      };
+      auto fetch_whole = [&](int it) {       // all moves of a tile at once (prologue)
+        if constexpr (!kFp8) {
           dma.begin(kv, s_rows, it * kTN, n_valid, tile_addr(it), wave, lane);
 #pragma unroll
           for (int j = 0; j < kDmaSteps; ++j) dma.step(j);
         } else {
-          stg.move_tile(kv, s_rows, it * kTN, n_valid, s_tile[it & (kSlots - 1)], tid);
+          pipe_begin(it);
+#pragma unroll
+          for (int j = 0; j < Fp8Pipe::kSteps; ++j) pipe.step(j);
         }
       };
       // scores + probabilities of tile `it` into P buffer it & 1; `side` threads DMA issue
@@ -467,7 +531,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
         const uint32_t tile = tile_addr(it);
         const int my_valid = min(kTN, n_valid - it * kTN) - 16 * dh;   // valid tokens among my 16
         f32x4 sa[4], s[2];
-        tile_scores(tile, 16 * dh, qf, sa, lane, side);
+        tile_scores(tile, rope_addr(it), 16 * dh, qf, sa, lane, side);
         s[0] = sa[0] + sa[1];
         s[1] = sa[2] + sa[3];
         if constexpr (CAP) {
@@ -512,20 +576,32 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
       };
 
       // ---- prologue: tiles 0 and 1 go out at once, tile 2 rides on the scores of tile 0
-      if constexpr (FMT == SMLA_KV_BF16) {
-        // The moves go out as soon as the row list exists; Q may still be on its way.  Loads
-        // complete in issue order, so waiting for the moves below also waits for everything older.
-        for (int it = 0; it < min(n_tiles, 2); ++it) fetch_whole(it);
+      // The moves go out as soon as the row list exists; Q may still be on its way.  Loads
+      // complete in issue order, so waiting for the moves below also waits for everything older.
+      for (int it = 0; it < min(n_tiles, 2); ++it) fetch_whole(it);
+      if constexpr (!kFp8) {
         wait_dma(n_tiles > 1 ? 1 : 0);
-        // Tell the compiler that Q has arrived (it cannot see the wait above): otherwise it would
-        // wait for Q inside the first tile's MFMA stream, and with it for the moves issued there.
-#pragma unroll
-        for (int ks = 0; ks < kDqk / 32; ++ks) hw::wait_for_loads_of(qf[ks][0], qf[ks][1]);
       } else {
-        for (int it = 0; it < min(n_tiles, kSlots - 1); ++it) fetch_whole(it);
+        // fp8: convert tile 0, send for tile 2 (its raw block is free again), convert tile 1
+        // (a wavefront's lanes read raw chunks that other lanes of it fetched: wave_lds_order)
+        if (n_tiles > 1) hw::wait_vmcnt<Fp8Pipe::kSteps>(); else hw::wait_vmcnt<0>();
+        hw::wave_lds_order();
+        convert_begin(0);
+        cv.whole_tile();
+        if (n_tiles > 2) fetch_whole(2);
+        if (n_tiles > 1) {
+          if (n_tiles > 2) hw::wait_vmcnt<Fp8Pipe::kSteps>(); else hw::wait_vmcnt<0>();
+          hw::wave_lds_order();
+          convert_begin(1);
+          cv.whole_tile();
+        }
       }
+      // Tell the compiler that Q has arrived (it cannot see the waits above): otherwise it would
+      // wait for Q inside the first tile's MFMA stream, and with it for the moves issued there.
+#pragma unroll
+      for (int ks = 0; ks < kDqk / 32; ++ks) hw::wait_for_loads_of(qf[ks][0], qf[ks][1]);
       __syncthreads();                       // tile 0 landed
-      if (FMT == SMLA_KV_BF16 && n_tiles > 2) {
+      if (!kFp8 && n_tiles > 2) {
         dma.begin(kv, s_rows, 2 * kTN, n_valid, tile_addr(2), wave, lane);
         score_tile(0, [&](int ks) { if ((ks & 1) == 0) dma.step(ks >> 1); });
       } else {
@@ -533,37 +609,33 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
       }
 
       // ---- main loop: iterations that still have a tile to fetch (it + 3 < n_tiles, so tiles it+1
-      // and it+2 exist).  The fetch of tile it+3 rides on the score MFMAs of tile it+1, one DMA
+      // and it+2 exist).  The fetch of tile it+3 rides on the score MFMAs of tile it+1, one move
       // instruction every second k-step: early in the iteration (the data has the longest way
       // to go) but spaced out (measured: bursts and later issue are both slower).  Main loop and
       // tail are separate loops, each with one call site per MFMA block, so the accumulators
       // stay in place.
+      // fp8: the raw records of tile it+2 (sent for one iteration ago) are converted into the
+      // body that tile it-1 has left, in 16 slices under the P.V MFMAs of tile it.
       const int n_main = max(n_tiles - (kSlots - 1), 0);
       int it = 0;
       for (; it < n_main; ++it) {
-        // tile it+1 was issued two iterations ago; only tile it+2 is still outstanding
-        if constexpr (FMT == SMLA_KV_BF16) wait_dma(1);
-        __syncthreads();                     // P of tile `it` is published, tile it+1 landed, tile it-1 is consumed
-        if constexpr (FMT == SMLA_KV_BF16)
+        // bf16: tile it+1 was issued two iterations ago; only tile it+2 is still outstanding
+        if constexpr (!kFp8) wait_dma(1);
+        __syncthreads();                     // P of tile `it` is published, tile it+1 landed / converted, tile it-1 is consumed
+        if constexpr (!kFp8) {
           dma.begin(kv, s_rows, (it + kSlots - 1) * kTN, n_valid, tile_addr(it + kSlots - 1), wave, lane);
-        else {
-          fetch_whole(it + kSlots - 1);
-          // The staging above waits for its own loads; what makes that wait short is that the
-          // records are in L2 already: every thread touches one 128-byte line of the tile after
-          // (8 probes cover a 656-byte record wherever it starts) with a 4-byte load whose
-          // destination is a sink in LDS, so no register waits for it.
-          if (it + kSlots < n_tiles) {
-            const int e = min((it + kSlots) * kTN + (tid >> 3), n_valid - 1);
-            const uint8_t* line = kv + (size_t)s_rows[e] * kRowBytesFp8 + min((tid & 7) * 128, kRowBytesFp8 - 4);
-            const uint32_t sink = hw::lds_addr(&s_sink[0]);
-            hw::dma_b32(line, sink);
-          }
+        } else {
+          pipe_begin(it + 3);
+          convert_begin(it + 2);
         }
         // Tile it+1 is never the last one here, so it is full: no masking, and the reference is
         // fixed, so the softmax is straight-line vector code that is scheduled under the P.V MFMAs.
         f32x4 sa[4];
-        tile_scores(tile_addr(it + 1), 16 * dh, qf, sa, lane, [&](int ks) {
-          if constexpr (FMT == SMLA_KV_BF16) { if ((ks & 1) == 0) dma.step(ks >> 1); }
+        tile_scores(tile_addr(it + 1), rope_addr(it + 1), 16 * dh, qf, sa, lane, [&](int ks) {
+          if ((ks & 1) == 0) {
+            if constexpr (!kFp8) dma.step(ks >> 1);
+            else if ((ks >> 1) < Fp8Pipe::kSteps) pipe.step(ks >> 1);
+          }
         });
         // softmax of tile it+1 in 16 slices, one after each P.V MFMA of tile it
         f32x4 sv[2];
@@ -573,6 +645,15 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
         tile_accumulate<true>(tile_addr(it), lds_p + ((it & 1) * 2 + hg) * kPBytes, kDvHalf * dh, acc, lane,
                               [](int) {},
                               [&](int i) {
+          if constexpr (kFp8) {
+            // chunk k = i / 4 of the conversion: its two halves, its stores, and the next chunk's
+            // read three slices ahead of its first use.  The moves of tile it+3, just issued,
+            // stay in flight; everything older has landed after the wait.
+            if (i == 0) { hw::wait_vmcnt<Fp8Pipe::kSteps>(); hw::wave_lds_order(); cv.load(0); }
+            else if ((i & 3) == 1) cv.half(0);
+            else if ((i & 3) == 2) cv.half(1);
+            else if ((i & 3) == 3) { cv.store(i >> 2); if (i < 15) cv.load((i >> 2) + 1); }
+          }
           if (i < 2) {                       // slices 0, 1: score block, per-lane maximum, reference of head tile i
             // (per-lane maximum only: the overflow test does not need the row maximum, and a
             // maximum pass folds the lanes of a head together when it ends)
@@ -602,11 +683,19 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
         hw::lds_write_b64(pw, pw2[0]);
         hw::lds_write_b64(pw + 16 * kPStride, pw2[1]);
       }
-      // ---- tail: the last tiles, nothing left to fetch
+      // ---- tail: the last tiles, nothing left to fetch (fp8: tile it+2 may still await its conversion)
       for (; it < n_tiles; ++it) {
         const bool next = it + 1 < n_tiles;
-        if constexpr (FMT == SMLA_KV_BF16) { if (next) wait_dma(it + 2 < n_tiles ? 1 : 0); }
+        if constexpr (!kFp8) { if (next) wait_dma(it + 2 < n_tiles ? 1 : 0); }
         __syncthreads();
+        if constexpr (kFp8) {
+          if (it + 2 < n_tiles) {
+            hw::wait_vmcnt<0>();
+            hw::wave_lds_order();
+            convert_begin(it + 2);
+            cv.whole_tile();
+          }
+        }
         if (next) score_tile(it + 1, [](int) {});
         tile_accumulate<false>(tile_addr(it), lds_p + ((it & 1) * 2 + hg) * kPBytes, kDvHalf * dh, acc, lane, [](int) {}, [](int) {});
       }
@@ -644,36 +733,43 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // row at a time, 4 consecutive dv columns per lane, so everything below moves 16 bytes per
   // lane in 1 KB runs and per-row scalars are wave-uniform.
   __syncthreads();
+  // The lane's coordinates are taken afresh here: derived from the hardware's lane counter, they
+  // need not be carried through the main loop in registers (or parked in scratch) for this use.
+  const int lane_e = hw::lane_id(), tid_e = 64 * wave + lane_e;
+  const int g_e = lane_e >> 5, c32_e = lane_e & 31, l16_e = lane_e & 15, q4_e = lane_e >> 4;
+  const int head_e = head0 + c32_e;
+  const bool head_ok_e = head_e < p.n_heads;
   // the arrival ticket of the split merge is taken here, so that its round trip to memory
   // overlaps the staging below (the merge itself is described further down)
-  if (p.n_splits > 1 && tid == 0)
+  if (p.n_splits > 1 && tid_e == 0)
     s_nvalid = ws_arrive(p, p.counters + (size_t)t * n_hblocks + hb, ws_magic, p.n_splits, sp);
 #pragma unroll
   for (int ht = 0; ht < 2; ++ht) {
     float l = l_part[ht];
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
-    if (q4 == 0) { s_x[wave][16 * ht + l16] = l; s_m[wave][16 * ht + l16] = m_ref[ht]; }
+    if (q4_e == 0) { s_x[wave][16 * ht + l16_e] = l; s_m[wave][16 * ht + l16_e] = m_ref[ht]; }
   }
   __syncthreads();
-  const float m_run = s_m[wave][c32];
-  const float l_tot = s_x[wave][c32] + s_x[partner][c32];
+  const float m_run = s_m[wave][c32_e];
+  const float l_tot = s_x[wave][c32_e] + s_x[partner][c32_e];
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const float lse_nat = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
   constexpr int kStageStride = kDvHalf + 4;                        // floats per staged row (+16 B pad)
-  float* stage = reinterpret_cast<float*>(&s_tile[0][0]) + wave * 32 * kStageStride;
+  static_assert(4 * 32 * kStageStride * 4 <= kRingBytes, "the staged blocks must fit the ring area");
+  float* stage = reinterpret_cast<float*>(&s_ring[0]) + wave * 32 * kStageStride;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const int row = 8 * (r >> 2) + 4 * g + (r & 3);
+    const int row = 8 * (r >> 2) + 4 * g_e + (r & 3);
 #pragma unroll
-    for (int dt = 0; dt < kAccTiles; ++dt) stage[row * kStageStride + 32 * dt + c32] = acc[dt][r];
+    for (int dt = 0; dt < kAccTiles; ++dt) stage[row * kStageStride + 32 * dt + c32_e] = acc[dt][r];
   }
   __syncthreads();                                                 // staged blocks and scalar exchange are done
-  if (g == 0) s_x[wave][c32] = inv;                                // per-row normaliser
+  if (g_e == 0) s_x[wave][c32_e] = inv;                                // per-row normaliser
   hw::wave_lds_order();
   const int n_rows = max(0, min(32, p.n_heads - head0));           // head rows that exist (wave-uniform; 0: the whole head group lies past the last head)
-  const int col4 = kDvHalf * dh + 4 * lane;                        // this lane's 4 dv columns
-  auto staged = [&](int row) { return *reinterpret_cast<const float4*>(stage + row * kStageStride + 4 * lane); };
+  const int col4 = kDvHalf * dh + 4 * lane_e;                        // this lane's 4 dv columns
+  auto staged = [&](int row) { return *reinterpret_cast<const float4*>(stage + row * kStageStride + 4 * lane_e); };
   auto store_bf16x4 = [&](int row, float4 v) {
     uint2 w;
     w.x = pack_bf16(v.x, v.y);
@@ -681,7 +777,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + ((size_t)t * p.n_heads + head0 + row) * kDv + col4) = w;
   };
   if (p.n_splits == 1) {
-    if (dh == 0 && g == 0 && head_ok) p.lse[(size_t)t * p.n_heads + head] = lse_nat;
+    if (dh == 0 && g_e == 0 && head_ok_e) p.lse[(size_t)t * p.n_heads + head_e] = lse_nat;
     for (int row = 0; row < n_rows; ++row) {
       const float sc = s_x[wave][row];
       float4 v = staged(row);
@@ -706,12 +802,12 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   unsigned long long* word = p.counters + (size_t)t * n_hblocks + hb;
   const int role = s_nvalid;                                       // ticket taken at the top of the epilogue
   auto give_up = [&]() {                                           // the workspace was not what it should be: mark the rows
-    if (dh == 0 && g == 0 && head_ok) p.lse[(size_t)t * p.n_heads + head] = __uint_as_float(0x7fc00000u);
+    if (dh == 0 && g_e == 0 && head_ok_e) p.lse[(size_t)t * p.n_heads + head_e] = __uint_as_float(0x7fc00000u);
   };
   if (role == kRoleError) { give_up(); return; }
   if (role == kRolePublish) {
-    if (dh == 0 && g == 0 && head_ok)
-      __hip_atomic_store(&p.part_lse[((size_t)t * ns + sp) * p.n_heads + head], lse_nat, __ATOMIC_RELAXED,
+    if (dh == 0 && g_e == 0 && head_ok_e)
+      __hip_atomic_store(&p.part_lse[((size_t)t * ns + sp) * p.n_heads + head_e], lse_nat, __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
     float* o = p.part_out + (((size_t)t * ns + sp) * p.n_heads + head0) * kDv + col4;
     for (int row = 0; row < n_rows; ++row) {
@@ -722,19 +818,19 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     }
     hw::wait_vmcnt<0>();
     __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid_e == 0) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
   // last arrival: every other split holds a ticket, so it is running and will publish.  Wait for
   // all of them, then fold the normalised partials in split order with every product and sum
   // rounded on its own (no fused multiply-add): the result does not depend on which split
   // happened to arrive last.  Per-head scalars live in lane = head row c32.
-  if (tid == 0) s_redo = ws_wait_published(p, word, ns, sp) ? 0 : 1;
+  if (tid_e == 0) s_redo = ws_wait_published(p, word, ns, sp) ? 0 : 1;
   __syncthreads();
   if (s_redo != 0) { give_up(); return; }
   auto split_lse = [&](int i) {
     if (i == sp) return lse_nat;
-    return head_ok ? __hip_atomic_load(&p.part_lse[((size_t)t * ns + i) * p.n_heads + head], __ATOMIC_RELAXED,
+    return head_ok_e ? __hip_atomic_load(&p.part_lse[((size_t)t * ns + i) * p.n_heads + head_e], __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT)
                    : -INFINITY;
   };
@@ -744,14 +840,14 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   float w_sum = 0.f;
   for (int i = 0; i < ns; ++i) w_sum = __fadd_rn(w_sum, __expf(split_lse(i) - m_safe));      // exp(-inf) = 0
   const float rw = w_sum > 0.f ? 1.f / w_sum : 0.f;
-  if (dh == 0 && g == 0 && head_ok)
-    p.lse[(size_t)t * p.n_heads + head] = w_sum > 0.f ? m_all + __logf(w_sum) : -INFINITY;
+  if (dh == 0 && g_e == 0 && head_ok_e)
+    p.lse[(size_t)t * p.n_heads + head_e] = w_sum > 0.f ? m_all + __logf(w_sum) : -INFINITY;
   // my own block becomes its normalised partial: the very numbers a publisher would have stored
   for (int row = 0; row < 32; ++row) {
     const float sc = s_x[wave][row];
     float4 v = staged(row);
     v.x = __fmul_rn(v.x, sc); v.y = __fmul_rn(v.y, sc); v.z = __fmul_rn(v.z, sc); v.w = __fmul_rn(v.w, sc);
-    *reinterpret_cast<float4*>(stage + row * kStageStride + 4 * lane) = v;
+    *reinterpret_cast<float4*>(stage + row * kStageStride + 4 * lane_e) = v;
   }
   float* s_w = s_m[wave];                                          // per-row weight of the split being folded
                                                                    // (written and read by this wavefront only: its LDS accesses complete in order)
@@ -764,7 +860,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     for (int i = 0; i < ns; ++i) {
       const float wi = __fmul_rn(__expf(split_lse(i) - m_safe), rw);
       hw::wave_lds_order();
-      if (g == 0) s_w[c32] = wi;
+      if (g_e == 0) s_w[c32_e] = wi;
       hw::wave_lds_order();
       f32x4 v[16];
       if (i == sp) {
@@ -794,7 +890,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
       if (r0 + j < n_rows) store_bf16x4(r0 + j, make_float4(sum[j][0], sum[j][1], sum[j][2], sum[j][3]));
   }
   __syncthreads();
-  if (tid == 0) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+  if (tid_e == 0) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
 }
 
 template <int FMT, bool CAP>

@@ -258,16 +258,19 @@ uint8_t* lds_ptr(uint32_t addr, size_t bytes) {
 }
 
 void dma_issue(const void* src, uint32_t lds_dst, int bytes) {
-  if (bytes != 4 && bytes != 16) fail("dma of %d bytes per lane", bytes);
+  if (bytes != 0 && bytes != 4 && bytes != 16) fail("dma of %d bytes per lane", bytes);
   if (g_dma_eager) {
+    if (bytes == 0) return;
     memcpy(lds_ptr(lds_dst, bytes), src, bytes);
     return;
   }
   Fiber::Pending p;
   p.lds_dst = lds_dst;
   p.bytes = bytes;
-  memcpy(p.data, src, bytes);
-  lds_ptr(lds_dst, bytes);                           // bounds check at issue
+  if (bytes != 0) {                                  // 0: a lane that sits out a move of its wavefront (kept for the count)
+    memcpy(p.data, src, bytes);
+    lds_ptr(lds_dst, bytes);                         // bounds check at issue
+  }
   g_cur->dma.push_back(p);
 }
 
@@ -275,7 +278,8 @@ void dma_wait(int allowed_in_flight) {
   std::vector<Fiber::Pending>& q = g_cur->dma;
   const size_t keep = std::min(q.size(), (size_t)std::max(allowed_in_flight, 0));
   const size_t land = q.size() - keep;
-  for (size_t i = 0; i < land; ++i) memcpy(lds_ptr(q[i].lds_dst, q[i].bytes), q[i].data, q[i].bytes);
+  for (size_t i = 0; i < land; ++i)
+    if (q[i].bytes != 0) memcpy(lds_ptr(q[i].lds_dst, q[i].bytes), q[i].data, q[i].bytes);
   q.erase(q.begin(), q.begin() + land);
 }
 

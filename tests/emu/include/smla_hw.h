@@ -46,10 +46,16 @@ inline bf16x4 lds_read_tr16_b64(uint32_t a) {
 }
 inline bf16x4 lds_read_tr16_b64(const void* shared_object) { return lds_read_tr16_b64(emu::lds_addr(shared_object)); }
 
+inline int lane_id() { return emu::self()->lane; }
 inline void wave_lds_order() { emu::wave_rendezvous(nullptr, 0, 0x4c44534fu); }
 
 inline void dma_b128(const void* lane_src, uint32_t lds_base) {
   emu::dma_issue(lane_src, lds_base + 16u * (uint32_t)emu::self()->lane, 16);
+}
+template <int N>
+inline void dma_b128_first_lanes(const void* lane_src, uint32_t lds_base) {
+  if (emu::self()->lane < N) dma_b128(lane_src, lds_base);
+  else emu::dma_issue(nullptr, 0, 0);                // the wavefront's instruction still counts for this lane's waits
 }
 inline void dma_b128(uint32_t lane_off, uint64_t wave_base, uint32_t lds_base) {
   emu::dma_issue(reinterpret_cast<const void*>(wave_base + lane_off), lds_base + 16u * (uint32_t)emu::self()->lane, 16);
@@ -64,6 +70,7 @@ inline void wait_vmcnt() { emu::dma_wait(N); }
 // the lane's outstanding moves, which is what the callers' issue order guarantees on hardware)
 template <typename... T> inline void wait_for_loads_of(const T&...) { emu::dma_wait(0); }
 template <typename... T> inline void pin(T&...) {}
+inline void pin_uniform(uint32_t&) {}
 
 inline void shift_in_gt_u32(uint32_t& mask, uint32_t x, uint32_t y) { mask = 2u * mask + (x > y ? 1u : 0u); }
 inline void shift_in_eq_u32(uint32_t& mask, uint32_t x, uint32_t y) { mask = 2u * mask + (x == y ? 1u : 0u); }

@@ -105,6 +105,40 @@ def test_fp8_records(heads, n_splits):
     _check(cfg, out, lse)
 
 
+@pytest.mark.parametrize("topk,n_splits", [(1, 1), (31, 1), (32, 1), (33, 1), (64, 2), (65, 1), (96, 1), (97, 1), (128, 1),
+                                           (129, 2), (200, 3), (1030, 1), (2100, 2)])
+def test_many_heads_fp8_pipeline_at_every_tile_count(topk, n_splits):
+    """The raw-record pipeline of the many-heads kernel has a prologue for the first two tiles,
+    a steady state from the fourth tile on and a tail for the last three: lists of 1, 2, 3, 4 and 5
+    tiles, ragged and full, more than one chunk of 1024 entries, and splits."""
+    cfg, _ = _fp8_cfg(1, 40, 40, topk, pad_frac=0.0 if topk < 40 else 0.04)
+    out, lse = _forward_all_ways(cfg, n_splits)
+    _check(cfg, out, lse)
+
+
+def test_many_heads_fp8_redo_passes():
+    """Scores that outgrow the first tile's reference: the fp8 pipeline runs three times over the list."""
+    g = torch.Generator().manual_seed(11)
+    latent = (torch.randn((400, 576), generator=g) * 4.0).to(torch.bfloat16)
+    latent[:64] *= 0.01
+    rec = torch.zeros((400, 656), dtype=torch.uint8)
+    assert harness.lib().smla_kv_quantize_fp8(latent.data_ptr(), None, rec.data_ptr(), 400, 400, None) == 0
+    q = (torch.randn((2, 64, 576), generator=g) * 4.0).to(torch.bfloat16)
+    cfg = dict(q=q, kv_cache=rec, indices=torch.arange(200, dtype=torch.int32).repeat(2, 1), block_table=None, page_size=64,
+               sm_scale=576 ** -0.5, kv_format="fp8_e4m3_b128")
+    # The kernel multiplies bf16(float(e4m3) * scale).  With scores of +-50 that rounding alone moves
+    # a score by a few hundredths and, between two near-equal top scores, the output by percents; so
+    # here (and only here) the oracle is fed the rounded products, which pins the pipeline itself.
+    qn, kv_small, phys_small, _ = oracle_inputs(cfg)
+    kv_small = torch.from_numpy(np.asarray(kv_small, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+    ro, rl = oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfg["sm_scale"], 512)
+    assert float(np.abs(rl).max()) > 40.0                     # far beyond what the first tile's reference allows for
+    for ns in (1, 2):
+        out, lse = _forward_all_ways(cfg, ns)
+        assert max_abs(to_np(lse).reshape(rl.shape), rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
+        assert max_abs(to_np(out).reshape(ro.shape), ro) <= 1.2e-2 * max(1.0, float(np.abs(ro).max()))
+
+
 @pytest.fixture
 def wide_kernel(monkeypatch):
     """Routes many-heads bf16 launches to the 128-heads-per-workgroup kernel (opt-in until it is measured)."""

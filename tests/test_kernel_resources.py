@@ -1,5 +1,5 @@
 """CPU check of what the compiled gfx950 kernels occupy (hipcc cross-compiles without a GPU):
-every kernel's LDS fits the CU's 160 KB, and only the one kernel known to spill uses scratch.
+every kernel's LDS fits the CU's 160 KB, and only the kernels named below use scratch at all.
 A spill in any other kernel is a performance regression.  Loads issued from inline assembly into
 registers are banned outright: the compiler takes an asm output as written when the statement
 ends, while the load is still in flight, so any copy or spill it places before the wait reads
@@ -15,13 +15,11 @@ from flagtree_amd import build
 
 LDS_PER_CU = 160 * 1024
 # Kernels that may park registers in scratch memory OUTSIDE their inner loops (checked below):
-#  * the many-heads forward over an fp8 cache converts its tiles in registers next to 128
-#    accumulators and 72 Q registers; it parks values across its prologue,
 #  * the two-workgroups-per-CU fp8 kernel is capped at 256 registers and parks a few across the
 #    per-chunk set-up.
 #  * the 128-heads-per-workgroup kernel keeps 200 of its 256 registers for Q and accumulators; it
 #    parks values across the per-chunk set-up and while the accumulators drain in the epilogue.
-MAY_SPILL = ("fwd_tall_kernelILi1E", "fwd_few_fp8_kernel", "fwd_wide_kernel")
+MAY_SPILL = ("fwd_few_fp8_kernel", "fwd_wide_kernel")
 
 _cache = {}
 
