@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle
-from _util import max_abs, oracle_inputs, run_oracle, to_np
+from _util import check_random_shape, max_abs, oracle_inputs, random_shape_draw, run_oracle, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -68,7 +68,7 @@ def test_scalar_kernel_matches_oracle(dev):
     _check(cfg, out, lse, out_tol=2e-3, lse_tol=1e-5)      # out is rounded to bf16 once
 
 
-@pytest.mark.parametrize("heads", [16, 128])
+@pytest.mark.parametrize("heads", [16])               # (128 heads: test_gpu_x_unproven_kernels.py)
 def test_decode_fp8_reduced(dev, heads):
     from flagtree_amd import workloads
     cfg = workloads.decode_fp8(dev, batch=3, heads=heads, pages_per_seq=32, topk=512, pad_frac=0.03)
@@ -381,9 +381,13 @@ def test_decode_attention_fwd_dense(dev, H, page_size, fmt):
 
 
 @pytest.mark.parametrize("H,fmt,std,cap,min_diff", [(128, "bf16", 1.5, 2.0, 0.5), (16, "bf16", 1.5, 2.0, 0.5),
-                                                    (16, "fp8_e4m3_b128", 1.5, 2.0, 0.5), (64, "fp8_e4m3_b128", 0.5, 0.2, 0.01)])
+                                                    (16, "fp8_e4m3_b128", 1.5, 2.0, 0.5)])
 @pytest.mark.parametrize("splits", [1, 2])
 def test_decode_attention_fwd_logit_cap(dev, H, fmt, std, cap, min_diff, splits):
+    check_logit_cap(dev, H, fmt, std, cap, min_diff, splits)
+
+
+def check_logit_cap(dev, H, fmt, std, cap, min_diff, splits):
     """logit_cap * tanh(score / logit_cap) before the softmax (reference test_accuracy_musa_vllm_mla.py:299-302);
     inputs scaled so that raw scores reach several times the cap.  (The many-heads kernel rounds
     dequantised fp8 values to bf16 when it stages them, an error that grows with the square of the
@@ -469,50 +473,10 @@ def test_forward_replays_from_a_hip_graph(dev):
 def test_random_shapes_against_oracle(dev, seed):
     """Seeded draws over head counts, list lengths, page sizes, tokens per sequence, split counts,
     padding patterns, page tables with holes and both cache formats (small enough for the host oracle)."""
-    import flagtree_amd as ft
-    rng = np.random.default_rng(4000 + seed)
-    g = torch.Generator().manual_seed(4000 + seed)
-    heads = int(rng.choice([1, 7, 16, 17, 32, 33, 64, 65, 127, 128]))
-    topk = int(rng.choice([1, 31, 32, 33, 100, 257, 1024, 1100, 2300]))
-    page_size = int(rng.choice([1, 16, 64]))
-    tokens_per_seq = int(rng.choice([1, 3]))
-    batch = int(rng.choice([1, 2, 5]))
-    fmt = "fp8_e4m3_b128" if rng.random() < 0.35 else "bf16"
-    n_splits = [None, 1, 2, 3, 5][int(rng.integers(5))]
-    paged = rng.random() < 0.7
-    ctx = int(rng.choice([64, 300, 2400]))                             # logical positions per sequence
-    lat = (torch.randn((batch * ctx + 128, 576), generator=g) * float(rng.choice([0.05, 0.2]))).to(torch.bfloat16)
-    if paged:
-        pages_per_seq = -(-ctx // page_size)
-        n_pages = batch * pages_per_seq + 3
-        kv_rows = n_pages * page_size
-        lat = (torch.randn((kv_rows, 576), generator=g) * 0.1).to(torch.bfloat16)
-        bt = torch.randperm(n_pages, generator=g)[:batch * pages_per_seq].to(torch.int32).view(batch, pages_per_seq)
-        if pages_per_seq > 2 and rng.random() < 0.5:
-            bt[0, 1] = -1                                               # a hole: its positions are masked
-        hi = pages_per_seq * page_size + (3 if rng.random() < 0.3 else 0)   # a few positions past the table
-    else:
-        bt = None
-        hi = lat.shape[0] + (2 if rng.random() < 0.3 else 0)
-    T = batch * tokens_per_seq
-    idx = torch.from_numpy(rng.integers(0, hi, size=(T, topk)).astype(np.int32))
-    pad = rng.random((T, topk)) < float(rng.choice([0.0, 0.1, 0.6]))
-    idx[torch.from_numpy(pad)] = -1
-    if rng.random() < 0.3:
-        idx[0, topk // 2:] = -1                                        # tail padding
-    if T > 1 and rng.random() < 0.3:
-        idx[1, :] = -1                                                 # a token with nothing to attend to
-    q = (torch.randn((batch, tokens_per_seq, heads, 576), generator=g) * 0.1).to(torch.bfloat16)
-    kv = lat.to(dev) if fmt == "bf16" else ft.quantize_kv_fp8(lat.to(dev))
-    if paged:
-        kv = kv.view(-1, page_size, kv.shape[-1])
-    cfg = dict(q=q.to(dev), kv_cache=kv, indices=idx.view(batch, tokens_per_seq, topk).to(dev),
-               block_table=bt.to(dev) if bt is not None else None, page_size=page_size, sm_scale=576 ** -0.5, kv_format=fmt)
-    out, lse = _fwd(cfg, n_splits=n_splits)
-    _check(cfg, out, lse)
-    so, sl = ft.sparse_mla_fwd_scalar(cfg["q"], cfg["kv_cache"], cfg["indices"], cfg["sm_scale"], 512,
-                                      block_table=cfg["block_table"], page_size=page_size, kv_format=fmt)
-    assert max_abs(to_np(out), to_np(so)) <= 1e-2 and max_abs(to_np(lse), to_np(sl)) <= 1e-3
+    draw = random_shape_draw(4000 + seed)
+    if draw["kv_format"] != "bf16" and draw["heads"] > 32:
+        pytest.skip("many heads over an fp8 cache: runs in test_gpu_x_unproven_kernels.py")
+    check_random_shape(draw, dev, _fwd, _check)
 
 
 @pytest.mark.parametrize("heads", [16, 128])
@@ -664,128 +628,3 @@ def test_properties_at_full_fp8_decode_size(dev):
     assert (out[:8].float() - so.float()).abs().max().item() <= OUT_TOL
     assert (lse[:8] - sl).abs().max().item() <= LSE_TOL
     _check(dict(sub, q=sub["q"][:2], indices=sub["indices"][:2], block_table=sub["block_table"][:2]), out[:2], lse[:2])
-
-
-# ---- the two-workgroups-per-CU fp8 kernel (opt-in until it has been measured) -------------------
-
-@pytest.fixture
-def few_fp8_kernel(monkeypatch):
-    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
-
-
-@pytest.mark.parametrize("heads,n_splits,topk", [(16, 1, 512), (16, 2, 512), (8, 3, 300), (30, 2, 700), (16, None, 2048)])
-def test_column_split_fp8_kernel_against_oracle(dev, few_fp8_kernel, heads, n_splits, topk):
-    from flagtree_amd import workloads
-    cfg = workloads.decode_fp8(dev, batch=5, heads=heads, pages_per_seq=40, topk=topk, pad_frac=0.03)
-    out, lse = _fwd(cfg, n_splits=n_splits)
-    _check(cfg, out, lse)
-
-
-def test_column_split_fp8_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch):
-    """Full fp8 decode size: the two kernels agree to the bar (they sum in different orders), and a
-    slice of the batch agrees with the oracle."""
-    from flagtree_amd import workloads
-    cfg = workloads.decode_fp8(dev)
-    out0, lse0 = _fwd(cfg)
-    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
-    out1, lse1 = _fwd(cfg)
-    torch.cuda.synchronize()
-    assert not torch.equal(out0, out1)                       # it really is the other kernel
-    assert max_abs(to_np(out1), to_np(out0)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse0)) <= 1e-4
-    sub = dict(cfg, q=cfg["q"][:4], indices=cfg["indices"][:4], block_table=cfg["block_table"][:4])
-    ro, rl = run_oracle(sub)
-    assert max_abs(to_np(out1[:4]).reshape(4, 16, 512), ro) <= OUT_TOL and max_abs(to_np(lse1[:4]).reshape(4, 16), rl) <= LSE_TOL
-
-
-def test_column_split_fp8_kernel_edge_cases_and_dense(dev, few_fp8_kernel):
-    import flagtree_amd as ft
-    g = torch.Generator().manual_seed(7)
-    latent = (torch.randn((300, 576), generator=g) * 0.1).to(torch.bfloat16).to(dev)
-    rec = ft.quantize_kv_fp8(latent)
-    q = (torch.randn((6, 16, 576), generator=g) * 0.1).to(torch.bfloat16).to(dev)
-    idx = torch.full((6, 70), -1, dtype=torch.int32)
-    idx[1, 33] = 5
-    idx[2, :] = torch.randperm(300, generator=g)[:70].to(torch.int32)
-    idx[3, :35] = 17
-    idx[4, ::2] = torch.arange(35, dtype=torch.int32)
-    idx[5, 0] = 299
-    idx[5, 1] = 300
-    cfg = dict(q=q, kv_cache=rec, indices=idx.to(dev), block_table=None, page_size=64, sm_scale=576 ** -0.5,
-               kv_format="fp8_e4m3_b128")
-    for ns in (1, 2):
-        out, lse = _fwd(cfg, n_splits=ns)
-        _check(cfg, out, lse)
-        assert (to_np(out)[0] == 0).all() and np.isneginf(to_np(lse)[0]).all()
-    # dense decode with a logit cap through the same kernel
-    B, L, page_size, cap = 3, 700, 64, 0.02
-    lens = torch.tensor([L, 3, 300], dtype=torch.int32)
-    n_pages = -(-L // page_size)
-    req = torch.randperm(2 * B * n_pages, generator=g)[:B * n_pages].to(torch.int32).view(B, n_pages)
-    lat = (torch.randn((2 * B * n_pages * page_size, 576), generator=g) * 0.1).to(torch.bfloat16)
-    k_buffer = ft.quantize_kv_fp8(lat.to(dev)).view(-1, page_size, 656)
-    qd = (torch.randn((B, 16, 576), generator=g) * 0.1).to(torch.bfloat16)
-    o, lse = ft.decode_attention_fwd(qd.to(dev), k_buffer, None, None, req.to(dev), lens.to(dev), None, 2, 576 ** -0.5,
-                                     page_size, logit_cap=cap)
-    max_len = n_pages * page_size
-    idxd = torch.arange(max_len, dtype=torch.int32).repeat(B, 1)
-    idxd[idxd >= lens[:, None]] = -1
-    cfgd = {"q": qd.view(B, 1, 16, 576), "indices": idxd.view(B, 1, max_len), "kv_cache": k_buffer, "block_table": req,
-            "page_size": page_size, "kv_format": "fp8_e4m3_b128", "sm_scale": 576 ** -0.5}
-    qn, kv_small, phys_small, _ = oracle_inputs(cfgd)
-    wo, wl = oracle.sparse_mla_fwd(qn, kv_small, phys_small, cfgd["sm_scale"], 512, logit_cap=cap)
-    assert max_abs(to_np(lse), wl.reshape(B, 16)) <= 1e-3 and max_abs(to_np(o), wo.reshape(B, 16, 512)) <= 1e-2
-
-
-# ---- the 128-heads-per-workgroup bf16 kernel (opt-in until it has been measured) ----------------
-
-@pytest.fixture
-def wide_kernel(monkeypatch):
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")
-
-
-@pytest.mark.parametrize("heads,n_splits,topk", [(128, 1, 512), (128, 2, 512), (64, 3, 300), (200, 2, 700), (128, None, 2048),
-                                                 (65, 3, 200)])
-def test_128_heads_kernel_against_oracle(dev, wide_kernel, heads, n_splits, topk):
-    from flagtree_amd import workloads
-    cfg = workloads.decode_bf16(dev, batch=5, heads=heads, pages_per_seq=40, topk=topk, pad_frac=0.03)
-    out, lse = _fwd(cfg, n_splits=n_splits)
-    _check(cfg, out, lse)
-
-
-def test_128_heads_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch):
-    """Headline decode size: the two kernels agree to the bar (they sum in different orders), and a
-    slice of the batch agrees with the oracle."""
-    from flagtree_amd import workloads
-    cfg = workloads.decode_bf16(dev)
-    out0, lse0 = _fwd(cfg)
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")
-    out1, lse1 = _fwd(cfg)
-    torch.cuda.synchronize()
-    assert not torch.equal(out0, out1)                       # it really is the other kernel
-    assert max_abs(to_np(out1), to_np(out0)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse0)) <= 1e-4
-    sub = dict(cfg, q=cfg["q"][:2], indices=cfg["indices"][:2], block_table=cfg["block_table"][:2])
-    ro, rl = run_oracle(sub)
-    H = cfg["q"].shape[-2]
-    assert max_abs(to_np(out1[:2]).reshape(2, H, 512), ro) <= OUT_TOL and max_abs(to_np(lse1[:2]).reshape(2, H), rl) <= LSE_TOL
-
-
-def test_128_heads_kernel_prefill_and_redo(dev, wide_kernel):
-    from flagtree_amd import workloads
-    cfg = workloads.prefill_causal_bf16(dev, tokens=300, heads=128, topk=256)
-    out, lse = _fwd(cfg)
-    rows = slice(130, 170)                                   # lists of 131..170 entries: more than one chunk of 128
-    sub = dict(cfg, q=cfg["q"][:, rows], indices=cfg["indices"][:, rows])
-    ro, rl = run_oracle(sub)
-    assert max_abs(to_np(out[:, rows]).reshape(ro.shape), ro) <= OUT_TOL
-    assert max_abs(to_np(lse[:, rows]).reshape(rl.shape), rl) <= LSE_TOL
-    g = torch.Generator().manual_seed(3)
-    kv = (torch.randn((400, 576), generator=g) * 4.0).to(torch.bfloat16)
-    kv[:64] *= 0.01
-    q = (torch.randn((2, 128, 576), generator=g) * 4.0).to(torch.bfloat16)
-    cfg = dict(q=q.to(dev), kv_cache=kv.to(dev), indices=torch.arange(200, dtype=torch.int32).repeat(2, 1).to(dev),
-               block_table=None, page_size=64, sm_scale=576 ** -0.5, kv_format="bf16")
-    ro, rl = run_oracle(cfg)
-    for ns in (1, 2):
-        out, lse = _fwd(cfg, n_splits=ns)
-        assert max_abs(to_np(lse).reshape(rl.shape), rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
-        assert max_abs(to_np(out).reshape(ro.shape), ro) <= 1.2e-2 * max(1.0, float(np.abs(ro).max()))
