@@ -110,6 +110,14 @@ def decode_fp8(device="cuda", seed=1004, batch=128, heads=16, pages_per_seq=2048
                 kv_format="fp8_e4m3_b128", name="decode_fp8")
 
 
+def decode_fp8_h128(device="cuda", seed=1006):
+    """The headline decode's shape (batch 64, 128 heads, top-k 2048 with 5 % padding, 65 536-token
+    contexts) over an fp8 cache: the many-heads kernel's fp8 path."""
+    cfg = decode_fp8(device, seed=seed, batch=64, heads=128, pages_per_seq=1024, topk=2048, pad_frac=0.05)
+    cfg["name"] = "decode_fp8_h128"
+    return cfg
+
+
 def gemm_rs_shard(device="cuda", seed=1005, m=8192, k=2048, n=7168, n_chunks=8):
     gd = _gen(device, seed)
     x = (torch.randn((m, k), generator=gd, device=device) * 0.02).to(torch.bfloat16)
