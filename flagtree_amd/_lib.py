@@ -72,3 +72,15 @@ def check(rc, what):
     if -10 < rc < 0:
         raise ValueError(msg)
     raise RuntimeError(msg)
+
+
+def on_device(t):
+    """True for a tensor in GPU memory.  The one place the wrappers ask (there is no CPU path)."""
+    return t.is_cuda
+
+
+def stream_handle(device):
+    """The caller's current stream on `device` as the hipStream_t the C ABI takes."""
+    import torch
+    return torch.cuda.current_stream(device).cuda_stream
+

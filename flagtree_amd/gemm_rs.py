@@ -18,7 +18,7 @@ def gemm_rs_local(x, w, partial=None, n_chunks=8, out=None):
         raise ValueError("x and w must be bfloat16")
     if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[0]:
         raise ValueError("x must be [M, K] and w [K, N]")
-    if not x.is_cuda:
+    if not _lib.on_device(x):
         raise ValueError("gemm_rs_local needs device tensors (there is no CPU path)")
     M, K = x.shape
     N = w.shape[1]
@@ -36,6 +36,6 @@ def gemm_rs_local(x, w, partial=None, n_chunks=8, out=None):
     lib = _lib.load()
     rc = lib.smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), partial.data_ptr() if partial is not None else None,
                                 out.data_ptr(), M, N, K, n_chunks, (M // n_chunks) * N,
-                                torch.cuda.current_stream(x.device).cuda_stream)
+                                _lib.stream_handle(x.device))
     _lib.check(rc, "smla_gemm_rs_local")
     return out

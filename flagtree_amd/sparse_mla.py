@@ -19,7 +19,7 @@ _FORMATS = {"bf16": _lib.SMLA_KV_BF16, "fp8_e4m3_b128": _lib.SMLA_KV_FP8_B128, "
 
 
 def _stream(t):
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return _lib.stream_handle(t.device)
 
 
 _I32_MAX = 2 ** 31 - 1
@@ -77,7 +77,7 @@ def _normalise(q, kv_cache, indices, d_v, block_table, kv_format, per_sequence=N
     if indices.dtype not in (torch.int32, torch.int64):
         raise ValueError("indices must be int32 or int64")
     for name, t in (("q", q), ("kv_cache", kv_cache), ("indices", indices)):
-        if not t.is_cuda:
+        if not _lib.on_device(t):
             raise ValueError(f"{name} must be a device tensor (there is no CPU path)")
     idx2 = _indices_i32(indices.reshape(T, K))
     if not idx2.is_contiguous():
@@ -102,7 +102,7 @@ def _normalise(q, kv_cache, indices, d_v, block_table, kv_format, per_sequence=N
     if block_table is not None:
         if block_table.dim() != 2 or block_table.shape[0] != B:
             raise ValueError("block_table must be [B, max_pages]")
-        if block_table.dtype != torch.int32 or not block_table.is_cuda:
+        if block_table.dtype != torch.int32 or not _lib.on_device(block_table):
             raise ValueError("block_table must be an int32 device tensor")
         block_table = block_table.contiguous()
     out_shape = (B, S, H, D_V) if q.dim() == 4 else (T, H, D_V)
@@ -139,7 +139,7 @@ def workspace_status(workspace):
 
 
 def _check_workspace(workspace, need, device):
-    if not isinstance(workspace, torch.Tensor) or not workspace.is_cuda or workspace.device != device:
+    if not isinstance(workspace, torch.Tensor) or not _lib.on_device(workspace) or workspace.device != device:
         raise ValueError("workspace must be a tensor on the inputs' device (see make_workspace)")
     if workspace.dtype != torch.uint8 or not workspace.is_contiguous():
         raise ValueError("workspace must be a contiguous uint8 tensor (see make_workspace)")
@@ -152,7 +152,7 @@ def _default_workspace(n_bytes, device):
     # the arrival words and partials; launches on different streams may overlap and must not.
     # A workspace that has to grow is replaced; the old tensor goes back to torch's allocator,
     # which keeps it away from other streams until this stream's queued work is done.
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    key = (device, _lib.stream_handle(device))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < n_bytes:
         ws = make_workspace(n_bytes, device)
@@ -243,7 +243,7 @@ def gather_rows(kv_cache, indices, *, block_table=None, page_size=64, tokens_per
     """Translate + mask + gather only.  kv_cache [..., W] any dtype (row = W elements, a multiple
     of 16 bytes); indices [T, topk].  Returns (phys int32 [T, topk] with -1 = masked,
     rows [T, topk, W] with zero rows where masked, or None)."""
-    if not kv_cache.is_cuda or not indices.is_cuda:
+    if not _lib.on_device(kv_cache) or not _lib.on_device(indices):
         raise ValueError("gather_rows needs device tensors (there is no CPU path)")
     kv2 = kv_cache.reshape(-1, kv_cache.shape[-1]).contiguous()
     if indices.dtype not in (torch.int32, torch.int64):
@@ -254,7 +254,7 @@ def gather_rows(kv_cache, indices, *, block_table=None, page_size=64, tokens_per
     phys = torch.empty((T, K), dtype=torch.int32, device=kv2.device)
     rows = torch.empty((T, K, kv2.shape[1]), dtype=kv2.dtype, device=kv2.device) if with_rows else None
     if block_table is not None:
-        if block_table.dtype != torch.int32 or not block_table.is_cuda:
+        if block_table.dtype != torch.int32 or not _lib.on_device(block_table):
             raise ValueError("block_table must be an int32 device tensor")
         block_table = block_table.contiguous()
     lib = _lib.load()
@@ -270,7 +270,7 @@ def gather_rows(kv_cache, indices, *, block_table=None, page_size=64, tokens_per
 
 def merge_splits(part_out, part_lse):
     """part_out fp32 [T, n_splits, H, 512], part_lse fp32 [T, n_splits, H] -> (out bf16 [T, H, 512], lse [T, H])."""
-    if not part_out.is_cuda:
+    if not _lib.on_device(part_out):
         raise ValueError("merge_splits needs device tensors (there is no CPU path)")
     T, ns, H, dv = part_out.shape
     part_out = part_out.contiguous().float()
@@ -286,7 +286,7 @@ def merge_splits(part_out, part_lse):
 def quantize_kv_fp8(latent, records=None, slot=None):
     """KV-cache writer for the fp8 format: latent bf16 [N, 576] -> uint8 records [rows, 656].
     ``slot`` int64 [N] names the destination row of each latent row (negative = skip)."""
-    if not latent.is_cuda:
+    if not _lib.on_device(latent):
         raise ValueError("quantize_kv_fp8 needs device tensors (there is no CPU path)")
     if latent.dtype != torch.bfloat16 or latent.shape[-1] != D_QK:
         raise ValueError("latent must be bf16 [..., 576]")
@@ -314,7 +314,7 @@ def reshape_and_cache(latent, kv_cache, slot_mapping, kv_format="bf16"):
     [..., 576] ("bf16") or uint8 [..., 656] records ("fp8_e4m3_b128", quantised on the way in);
     ``slot_mapping`` int64 [num_tokens] = page * page_size + offset, negative = skip.  Returns None,
     like the reference (the cache is updated in place)."""
-    if not latent.is_cuda or not kv_cache.is_cuda or not slot_mapping.is_cuda:
+    if not _lib.on_device(latent) or not _lib.on_device(kv_cache) or not _lib.on_device(slot_mapping):
         raise ValueError("reshape_and_cache needs device tensors (there is no CPU path)")
     if latent.dtype != torch.bfloat16 or latent.shape[-1] != D_QK:
         raise ValueError("latent must be bf16 [..., 576]")
@@ -345,7 +345,7 @@ def topk_indices(scores, k, context_lens=None):
     (f32 [..., N]) among its first ``context_lens[row]`` entries (default N), ascending, -1 padded.
     Ties at the k-th value go to the lower index.  The reference only has ``topk`` as a language
     primitive returning values (/root/reference/third_party/metax/python/triton/language/standard.py:443)."""
-    if not scores.is_cuda:
+    if not _lib.on_device(scores):
         raise ValueError("topk_indices needs device tensors (there is no CPU path)")
     if scores.dtype != torch.float32:
         raise ValueError("scores must be float32")
@@ -359,7 +359,7 @@ def topk_indices(scores, k, context_lens=None):
     cl = None
     if context_lens is not None:
         cl = context_lens.reshape(-1).to(torch.int32).contiguous()
-        if cl.shape[0] != rows or not cl.is_cuda:
+        if cl.shape[0] != rows or not _lib.on_device(cl):
             raise ValueError("context_lens needs one device entry per row")
     out = torch.empty((rows, k), dtype=torch.int32, device=scores.device)
     rc = _lib.load().smla_topk_indices(s2.data_ptr(), cl.data_ptr() if cl is not None else None, out.data_ptr(),
@@ -397,7 +397,7 @@ def decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len, attn
     if q.dim() != 3 or q.shape[-1] != D_QK:
         raise ValueError("q must be [B, H, 576]")
     for name, t in (("q", q), ("k_buffer", k_buffer), ("req_to_token", req_to_token), ("b_seq_len", b_seq_len)):
-        if not t.is_cuda:
+        if not _lib.on_device(t):
             raise ValueError(f"{name} must be a device tensor (there is no CPU path)")
     if v_buffer is not None and (v_buffer.data_ptr() != k_buffer.data_ptr() or v_buffer.shape[-1] != D_V or
                                  v_buffer.dtype != k_buffer.dtype or v_buffer.dim() != k_buffer.dim() or

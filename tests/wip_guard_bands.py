@@ -41,7 +41,8 @@ class Banded:
 
 
 def _stream(dev):
-    return torch.cuda.current_stream(dev).cuda_stream
+    from flagtree_amd import _lib
+    return _lib.stream_handle(dev)
 
 
 def _forward_banded(cfg, n_splits, dev):
@@ -119,7 +120,7 @@ def test_cache_writer_stays_inside_the_cache(dev, fmt, row_bytes):
     import flagtree_amd as ft
     from flagtree_amd import _lib
     g = torch.Generator(device=dev).manual_seed(17)
-    n_tok, cache_rows = 300, 257
+    n_tok, cache_rows = 290, 257
     latent = (torch.randn((n_tok, 576), generator=g, device=dev) * 0.3).to(torch.bfloat16)
     slots = torch.randperm(cache_rows + 40, generator=g, device=dev)[:n_tok].to(torch.int64) - 20   # some negative, some past the pool
     cache_b = Banded(cache_rows * row_bytes, dev, fill=0)
