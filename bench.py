@@ -43,8 +43,9 @@ def parse():
                     help="first run three plain 1 GiB device copies (known HBM traffic) so a rocprofv3 --pmc "
                          "run of this command holds a reference kernel to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
-    ap.add_argument("--wide", action="store_true",
-                    help="bf16 many-heads workloads on the 128-heads-per-workgroup kernel (sets FLAGTREE_SMLA_WIDE=1; opt-in until measured)")
+    ap.add_argument("--wide", type=int, nargs="?", const=1, default=0, choices=[0, 1, 2],
+                    help="bf16 many-heads workloads on a 128-heads-per-workgroup kernel (sets FLAGTREE_SMLA_WIDE; 1: eight wavefronts, "
+                         "2: a wavefront per 32 heads; opt-in until measured)")
     ap.add_argument("--few-fp8", action="store_true",
                     help="decode_fp8 on the two-workgroups-per-CU kernel (sets FLAGTREE_SMLA_FEW_FP8=1; opt-in until measured)")
     return ap.parse_args()
@@ -116,7 +117,7 @@ def main():
     if a.few_fp8:
         os.environ["FLAGTREE_SMLA_FEW_FP8"] = "1"
     if a.wide:
-        os.environ["FLAGTREE_SMLA_WIDE"] = "1"
+        os.environ["FLAGTREE_SMLA_WIDE"] = str(a.wide)
     import torch
     import flagtree_amd as ft
     from flagtree_amd import workloads
@@ -237,7 +238,7 @@ def main():
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = measured_traffic(a.workload)
     roof["traffic_source"] = TRAFFIC_NOTE
-    roof["kernel"] = ("fwd_wide_kernel" if a.wide and not hbm_bound else "fwd_tall_kernel") if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
+    roof["kernel"] = ({1: "fwd_wide_kernel", 2: "fwd_group_kernel"}[a.wide] if a.wide and fmt == "bf16" else "fwd_tall_kernel") if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
     roof["kernel_ms"] = kern_ms
     roof["other_bound"] = (dict(bound="hbm", achieved=nbytes / (kern_ms * 1e-3) / 1e9, peak=PEAK_HBM_GBS, unit="GB/s")
                            if not hbm_bound else

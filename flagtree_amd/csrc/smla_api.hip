@@ -28,12 +28,13 @@ int check_common(const void* q, const void* kv, const int32_t* indices, const vo
 // Kernels that have passed the parity checks but whose speed has not been measured on hardware
 // yet stay behind a switch until it has (read at every call): FLAGTREE_SMLA_FEW_FP8=1 sends few-heads launches over an
 // fp8 cache to the two-workgroups-per-CU kernel (smla_mfma_few_fp8.hip).  Read at every call.
-// FLAGTREE_SMLA_WIDE=1 sends many-heads launches over a bf16 cache to the 128-heads-per-workgroup
-// kernel (smla_mfma_wide.hip).
-bool wide_enabled() {
+// FLAGTREE_SMLA_WIDE=1 or 2 sends many-heads launches over a bf16 cache to a 128-heads-per-workgroup
+// kernel: 1 = eight wavefronts (smla_mfma_wide.hip), 2 = a wavefront per 32 heads (smla_mfma_group.hip).
+int wide_mode() {                            // 0: off
   const char* e = getenv("FLAGTREE_SMLA_WIDE");
-  return e != nullptr && e[0] == '1';
+  return e == nullptr ? 0 : (e[0] == '1' ? 1 : (e[0] == '2' ? 2 : 0));
 }
+bool wide_enabled() { return wide_mode() != 0; }
 
 bool few_fp8_enabled() {
   const char* e = getenv("FLAGTREE_SMLA_FEW_FP8");
@@ -194,7 +195,7 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
     p.part_out = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + SMLA_WS_COUNTER_BYTES);
     p.part_lse = p.part_out + (size_t)n_tokens * n_splits * n_heads * d_v;
   }
-  if (n_heads > 32 && kv_format == SMLA_KV_BF16 && wide_enabled()) return launch_fwd_wide(p, s);
+  if (n_heads > 32 && kv_format == SMLA_KV_BF16 && wide_enabled()) return wide_mode() == 2 ? launch_fwd_group(p, s) : launch_fwd_wide(p, s);
   if (n_heads > 32) return launch_fwd_tall(kv_format, p, s);
   if (kv_format == SMLA_KV_FP8_B128 && few_fp8_enabled()) return launch_fwd_few_fp8(p, s);
   return launch_fwd_short(kv_format, p, s);

@@ -199,7 +199,8 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
 int launch_fwd_scalar(int kv_format, const Params& p, hipStream_t s);
 int launch_fwd_tall(int kv_format, const Params& p, hipStream_t s);    // n_heads > 32 (logit cap: a second instantiation)
 int launch_fwd_short(int kv_format, const Params& p, hipStream_t s);   // n_heads <= 32
-int launch_fwd_wide(const Params& p, hipStream_t s);                   // n_heads > 32, bf16 rows, 128 heads per workgroup (opt-in)
+int launch_fwd_wide(const Params& p, hipStream_t s);                   // n_heads > 32, bf16 rows, 128 heads per workgroup, 8 wavefronts (opt-in)
+int launch_fwd_group(const Params& p, hipStream_t s);                  // n_heads > 32, bf16 rows, 128 heads per workgroup, a wavefront per 32 heads (opt-in)
 int launch_fwd_few_fp8(const Params& p, hipStream_t s);                // n_heads <= 32, fp8 records, two workgroups per CU (opt-in)
 int launch_merge(const float* part_out, const float* part_lse, void* out, float* lse,
                  int n_tokens, int n_heads, int d_v, int n_splits, hipStream_t s);

@@ -140,6 +140,10 @@ CASES = {
     "short_fp8_split": forward_case(lambda: fp8_cfg(2, 16, 4, 150), 2),
     "wide_bf16_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=2, heads=128, pages_per_seq=5, topk=200, pad_frac=0.06), 2,
                                     env={"FLAGTREE_SMLA_WIDE": "1"}),
+    "group_bf16_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=2, heads=128, pages_per_seq=5, topk=200, pad_frac=0.06), 2,
+                                      env={"FLAGTREE_SMLA_WIDE": "2"}),
+    "group_bf16_ragged": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=65, pages_per_seq=5, topk=90, pad_frac=0.06), 3,
+                                       env={"FLAGTREE_SMLA_WIDE": "2"}),
     "wide_bf16_ragged": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=65, pages_per_seq=5, topk=90, pad_frac=0.06), 3,
                                      env={"FLAGTREE_SMLA_WIDE": "1"}),
     "few_fp8_split": forward_case(lambda: fp8_cfg(2, 16, 4, 150), 2, env={"FLAGTREE_SMLA_FEW_FP8": "1"}),

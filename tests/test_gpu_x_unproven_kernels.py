@@ -135,9 +135,9 @@ def test_column_split_fp8_kernel_edge_cases_and_dense(dev, few_fp8_kernel):
 
 # ---- the 128-heads-per-workgroup bf16 kernel (opt-in until it has been measured) ----------------
 
-@pytest.fixture
-def wide_kernel(monkeypatch):
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")
+@pytest.fixture(params=["1", "2"], ids=["eight_wavefronts", "wavefront_per_head_group"])
+def wide_kernel(request, monkeypatch):
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", request.param)
 
 
 @pytest.mark.parametrize("heads,n_splits,topk", [(128, 1, 512), (128, 2, 512), (64, 3, 300), (200, 2, 700), (128, None, 2048),
@@ -149,13 +149,14 @@ def test_128_heads_kernel_against_oracle(dev, wide_kernel, heads, n_splits, topk
     _check(cfg, out, lse)
 
 
-def test_128_heads_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch):
+@pytest.mark.parametrize("mode", ["1", "2"])
+def test_128_heads_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch, mode):
     """Headline decode size: the two kernels agree to the bar (they sum in different orders), and a
     slice of the batch agrees with the oracle."""
     from flagtree_amd import workloads
     cfg = workloads.decode_bf16(dev)
     out0, lse0 = _fwd(cfg)
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", mode)
     out1, lse1 = _fwd(cfg)
     torch.cuda.synchronize()
     assert not torch.equal(out0, out1)                       # it really is the other kernel

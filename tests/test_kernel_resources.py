@@ -19,7 +19,9 @@ LDS_PER_CU = 160 * 1024
 #    per-chunk set-up.
 #  * the 128-heads-per-workgroup kernel keeps 200 of its 256 registers for Q and accumulators; it
 #    parks values across the per-chunk set-up and while the accumulators drain in the epilogue.
-MAY_SPILL = ("fwd_few_fp8_kernel", "fwd_wide_kernel")
+#  * the wavefront-per-head-group kernel holds 144 Q and 256 accumulator registers; it parks values
+#    across the per-chunk set-up and in the epilogue's merge.
+MAY_SPILL = ("fwd_few_fp8_kernel", "fwd_wide_kernel", "fwd_group_kernel")
 
 _cache = {}
 
@@ -59,10 +61,16 @@ def _scratch_in_inner_loops(asm_text):
     basic blocks with the loop they belong to; an innermost loop's header says 'Inner Loop Header'."""
     out, kernel, inner, block_loop = {}, None, set(), None
     lines = asm_text.splitlines()
+    last_label = None
     for line in lines:                                    # first pass: the innermost loop headers
-        m = re.match(r"^(\.LBB\d+_\d+):.*This Inner Loop Header", line)
+        m = re.match(r"^(\.LBB\d+_\d+):", line)
         if m:
-            inner.add(m.group(1)[2:])                     # 'BB3_195'
+            last_label = m.group(1)[2:]                   # 'BB3_195'
+        elif not re.match(r"^\s+;", line):
+            last_label = None if line.strip() else last_label
+        # (a nested loop's header carries the note on a continuation line under its 'Parent Loop' lines)
+        if "This Inner Loop Header" in line and last_label:
+            inner.add(last_label)
     for line in lines:
         m = re.match(r"^(_Z\w+):", line)
         if m:
@@ -118,6 +126,8 @@ def test_one_wavefront_per_simd_kernels_use_the_whole_register_file():
     the 256 x 256 GEMM runs 16 wavefronts per workgroup, so 4 per SIMD, 128 registers each."""
     tall = _resource_usage("smla_mfma_tall.hip")
     assert all(u["Occupancy"] == 1 for u in tall.values()), tall
+    group = _resource_usage("smla_mfma_group.hip")
+    assert group and all(u["Occupancy"] == 1 and u["AGPRs"] == 256 for u in group.values()), group
     gemm = _resource_usage("gemm_rs.hip")
     big = [u for n, u in gemm.items() if "gemm_rs_big_kernel" in n]
     assert len(big) == 1 and big[0]["VGPRs"] + big[0]["AGPRs"] <= 128 and big[0]["LDS Size"] == 128 * 1024, big
