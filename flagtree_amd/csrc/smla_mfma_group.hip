@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   __shared__ __attribute__((aligned(1024))) uint8_t s_ring[kSlots * kTileBytes];   // swizzle xors need 1 KB alignment
   __shared__ int32_t s_rows[kChunk];
   __shared__ float s_inv[4][32];                                  // per-head normalisers (epilogue)
-  __shared__ float s_w[4][32];                                    // split merge: per-row weights of the round
+  __shared__ float s_w[4][4][16];                                 // split merge: [wavefront][split of the batch][row of the head tile] weights
   __shared__ int s_nvalid;
   __shared__ int s_cnt[4];
   __shared__ int s_redo;
@@ -581,7 +581,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   if (wave == 0 && lane_e == 0) s_redo = ws_wait_published(p, word, ns, sp) ? 0 : 1;
   __syncthreads();
   if (s_redo != 0) { give_up(); return; }
-  constexpr int kRound = 4;
+  constexpr int kRound = 4, kBatch = 4;
 #pragma unroll 1
   for (int ht = 0; ht < 2; ++ht) {
     const float own_lse = ht == 0 ? lse_nat[0] : lse_nat[1];      // (registers: the index must be a constant)
@@ -601,43 +601,58 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
     stage_tile(ht);
     const int rows_here = max(0, min(16, n_rows - 16 * ht));
 #pragma unroll 1
-    for (int r0 = 0; r0 < 16; r0 += kRound) {                      // kRound rows per round: 2 * kRound loads in flight per lane
+    for (int r0 = 0; r0 < 16; r0 += kRound) {
+      // Rounds of kRound rows; the splits are taken kBatch at a time, all their loads issued before
+      // the first is used (2 * kRound * kBatch = 32 sixteen-byte loads in flight per lane, 128 KB per
+      // workgroup: what the merge costs is the latency of these loads), then folded in split order.
       f32x4 sum[kRound][2];
 #pragma unroll
       for (int j = 0; j < kRound; ++j) { sum[j][0] = f32x4{0.f, 0.f, 0.f, 0.f}; sum[j][1] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll 1
-      for (int i = 0; i < ns; ++i) {
-        const float wi = __fmul_rn(__expf(split_lse(i) - m_safe), rw);   // lane (q4, l16): weight of row l16 of the tile
+      for (int i0 = 0; i0 < ns; i0 += kBatch) {
         hw::wave_lds_order();
-        if (q4_e == 0) s_w[wave][l16_e] = wi;
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {   // lane (q4, l16): weight of row l16 of the tile for split i0 + b
+          const float wi = i0 + b < ns ? __fmul_rn(__expf(split_lse(i0 + b) - m_safe), rw) : 0.f;
+          if (q4_e == 0) s_w[wave][b][l16_e] = wi;
+        }
         hw::wave_lds_order();
-        f32x4 v[kRound][2];
-        if (i == sp) {
+        f32x4 v[kBatch][kRound][2];
 #pragma unroll
-          for (int j = 0; j < kRound; ++j) {
-            const float4 a = staged(r0 + j, 0), b = staged(r0 + j, 1);
-            v[j][0] = f32x4{a.x, a.y, a.z, a.w};
-            v[j][1] = f32x4{b.x, b.y, b.z, b.w};
+        for (int b = 0; b < kBatch; ++b) {
+          const int i = i0 + b;
+          if (i < ns && i != sp && rows_here > r0) {
+            const hw::buffer_rsrc src = hw::make_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0 + 16 * ht) * kDv);
+#pragma unroll
+            for (int j = 0; j < kRound; ++j) {
+              const uint32_t off = (uint32_t)((min(r0 + j, rows_here - 1) * kDv + col8) * 4);
+              v[b][j][0] = hw::load_b128_agent(src, off);
+              v[b][j][1] = hw::load_b128_agent(src, off + 16);
+            }
+          } else if (i == sp) {
+#pragma unroll
+            for (int j = 0; j < kRound; ++j) {
+              const float4 a = staged(r0 + j, 0), c = staged(r0 + j, 1);
+              v[b][j][0] = f32x4{a.x, a.y, a.z, a.w};
+              v[b][j][1] = f32x4{c.x, c.y, c.z, c.w};
+            }
+          } else {                           // no such split, or rows past the last head: nothing to read, nothing stored
+#pragma unroll
+            for (int j = 0; j < kRound; ++j) { v[b][j][0] = f32x4{0.f, 0.f, 0.f, 0.f}; v[b][j][1] = f32x4{0.f, 0.f, 0.f, 0.f}; }
           }
-        } else if (rows_here > r0) {
-          const hw::buffer_rsrc src = hw::make_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0 + 16 * ht) * kDv);
-#pragma unroll
-          for (int j = 0; j < kRound; ++j) {
-            const uint32_t off = (uint32_t)((min(r0 + j, rows_here - 1) * kDv + col8) * 4);
-            v[j][0] = hw::load_b128_agent(src, off);
-            v[j][1] = hw::load_b128_agent(src, off + 16);
-          }
-        } else {                             // rows past the last head: nothing to read, nothing stored
-#pragma unroll
-          for (int j = 0; j < kRound; ++j) { v[j][0] = f32x4{0.f, 0.f, 0.f, 0.f}; v[j][1] = f32x4{0.f, 0.f, 0.f, 0.f}; }
         }
 #pragma unroll
-        for (int j = 0; j < kRound; ++j) {
-          const float rb = s_w[wave][r0 + j];
+        for (int b = 0; b < kBatch; ++b) {
+          if (i0 + b < ns) {
 #pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            sum[j][0][c] = __fadd_rn(sum[j][0][c], __fmul_rn(v[j][0][c], rb));
-            sum[j][1][c] = __fadd_rn(sum[j][1][c], __fmul_rn(v[j][1][c], rb));
+            for (int j = 0; j < kRound; ++j) {
+              const float rb = s_w[wave][b][r0 + j];
+#pragma unroll
+              for (int c = 0; c < 4; ++c) {
+                sum[j][0][c] = __fadd_rn(sum[j][0][c], __fmul_rn(v[b][j][0][c], rb));
+                sum[j][1][c] = __fadd_rn(sum[j][1][c], __fmul_rn(v[b][j][1][c], rb));
+              }
+            }
           }
         }
       }
