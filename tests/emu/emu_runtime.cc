@@ -257,6 +257,49 @@ uint8_t* lds_ptr(uint32_t addr, size_t bytes) {
   return reinterpret_cast<uint8_t*>(__start_emu_lds) + addr;
 }
 
+bool g_lds_profile = false;
+unsigned long long g_lds_stats[9] = {0};
+
+void lds_account(uint32_t addr, int bytes, int kind) {
+  if (!g_lds_profile) return;
+  const int par = wave_rendezvous(&addr, sizeof(addr), 0x4c424b30u + (uint32_t)kind);
+  Lane* me = self();
+  int first_live = 0;
+  while (first_live < kWave && !wave_lane_live(first_live)) ++first_live;
+  if (me->lane != first_live) return;                     // one lane does the sums for the wavefront
+  const int group = bytes >= 16 ? 16 : (bytes == 8 ? 32 : 64);
+  unsigned long long passes = 0, ideal = 0;
+  for (int g0 = 0; g0 < kWave; g0 += group) {
+    uint32_t words[64][4];                                // distinct word addresses seen per bank (small sets)
+    int n_words[64] = {0};
+    bool any = false;
+    for (int l = g0; l < g0 + group; ++l) {
+      if (!wave_lane_live(l)) continue;
+      any = true;
+      uint32_t a;
+      memcpy(&a, wave_slot(par, l), sizeof(a));
+      for (int w = 0; w < bytes / 4; ++w) {
+        const uint32_t word = a / 4 + w;
+        const int bank = word % 64;
+        bool seen = false;
+        for (int k = 0; k < n_words[bank] && k < 4; ++k) seen |= words[bank][k] == word;
+        if (!seen) {
+          if (n_words[bank] < 4) words[bank][n_words[bank]] = word;
+          n_words[bank]++;                                // (beyond four distinct words the count may overshoot: it is a conflict either way)
+        }
+      }
+    }
+    if (!any) continue;
+    int worst = 1;
+    for (int b = 0; b < 64; ++b) worst = std::max(worst, n_words[b]);
+    passes += worst;
+    ideal += 1;
+  }
+  g_lds_stats[3 * kind + 0] += 1;
+  g_lds_stats[3 * kind + 1] += passes;
+  g_lds_stats[3 * kind + 2] += ideal;
+}
+
 void dma_issue(const void* src, uint32_t lds_dst, int bytes) {
   if (bytes != 0 && bytes != 4 && bytes != 16) fail("dma of %d bytes per lane", bytes);
   if (g_dma_eager) {
@@ -343,4 +386,11 @@ void emu_set_dma_mode(int eager) { emu::g_dma_eager = eager; }
 void emu_set_block_order(unsigned seed) { emu::g_order_seed = seed; }
 unsigned long long emu_launch_count(void) { return emu::g_launches; }
 void emu_set_cu_count(int n) { emu::g_cu_count = n; }
+void emu_set_lds_profile(int on) {
+  emu::g_lds_profile = on != 0;
+  for (auto& v : emu::g_lds_stats) v = 0;
+}
+void emu_lds_profile(unsigned long long out[9]) {
+  for (int i = 0; i < 9; ++i) out[i] = emu::g_lds_stats[i];
+}
 }

@@ -55,6 +55,12 @@ uint8_t* lds_ptr(uint32_t addr, size_t bytes);       // bounds-checked
 void dma_issue(const void* src, uint32_t lds_dst, int bytes);
 void dma_wait(int allowed_in_flight);
 
+// LDS bank accounting (off unless emu_set_lds_profile(1)): a wavefront-wide LDS access by 32-bit
+// address, `bytes` per lane, is a rendezvous of the wavefront; the access is priced as the hardware
+// serves it: 16-byte accesses 16 lanes at a time, 8-byte accesses 32 lanes at a time, 64 banks of
+// 4 bytes, one pass per distinct word a bank is asked for.  kind: 0 read, 1 transposing read, 2 write.
+void lds_account(uint32_t addr, int bytes, int kind);
+
 void launch(Dim3 grid, Dim3 block, const std::function<void()>& body);
 int cu_count();                       // what the stand-in device reports as its number of compute units
 
@@ -68,4 +74,7 @@ void emu_set_dma_mode(int eager);        // 0: moves land at the wait (default),
 void emu_set_block_order(unsigned seed); // 0: ascending block ids, else a seeded shuffle
 unsigned long long emu_launch_count(void);
 void emu_set_cu_count(int n);            // before the library's first query (it caches the answer); default 256
+void emu_set_lds_profile(int on);        // 1: count bank passes of the kernels' addressed LDS accesses (slower); resets the counts
+// out[3 * kind + 0] wavefront instructions, + 1 passes they took, + 2 passes a conflict-free access would take
+void emu_lds_profile(unsigned long long out[9]);
 }

@@ -33,6 +33,8 @@ def lib():
         l.emu_set_block_order.argtypes = [ctypes.c_uint]
         l.emu_launch_count.restype = ctypes.c_ulonglong
         l.emu_set_cu_count.argtypes = [ctypes.c_int]
+        l.emu_set_lds_profile.argtypes = [ctypes.c_int]
+        l.emu_lds_profile.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
         l.emu_set_cu_count(EMU_CUS)                      # before the library's first (cached) query
         _lib = l
     return _lib
@@ -42,6 +44,19 @@ def configure(dma_eager=False, block_order_seed=0):
     l = lib()
     l.emu_set_dma_mode(1 if dma_eager else 0)
     l.emu_set_block_order(block_order_seed)
+
+
+def lds_profile_start():
+    """Count bank passes of the kernels' addressed LDS accesses from now on (slower)."""
+    lib().emu_set_lds_profile(1)
+
+
+def lds_profile_stop():
+    """{'read' | 'read_tr' | 'write': (wavefront instructions, passes taken, passes without conflicts)}"""
+    out = (ctypes.c_ulonglong * 9)()
+    lib().emu_lds_profile(out)
+    lib().emu_set_lds_profile(0)
+    return {k: tuple(int(out[3 * i + j]) for j in range(3)) for i, k in enumerate(("read", "read_tr", "write"))}
 
 
 _FORMATS = {"bf16": 0, "fp8_e4m3_b128": 1, "f32": 2}

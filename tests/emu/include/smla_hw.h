@@ -17,18 +17,21 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 inline uint32_t lds_addr(const void* shared_object) { return emu::lds_addr(shared_object); }
 inline bf16x8 lds_read_b128(uint32_t a) {
   if (a & 15) emu::fail("ds_read_b128 at unaligned LDS address %u", a);
+  emu::lds_account(a, 16, 0);
   bf16x8 v;
   memcpy(&v, emu::lds_ptr(a, 16), 16);
   return v;
 }
 inline void lds_write_b64(uint32_t a, u32x2 v) {
   if (a & 7) emu::fail("ds_write_b64 at unaligned LDS address %u", a);
+  emu::lds_account(a, 8, 2);
   memcpy(emu::lds_ptr(a, 8), &v, 8);
 }
 // ds_read_b64_tr_b16: inside each group of 16 lanes, lane i receives element (i % 4) of the 8-byte
 // rows addressed by lanes (i / 4), (i / 4) + 4, (i / 4) + 8, (i / 4) + 12 of the group.
 inline bf16x4 lds_read_tr16_b64(uint32_t a) {
   if (a & 7) emu::fail("ds_read_b64_tr_b16 at unaligned LDS address %u", a);
+  emu::lds_account(a, 8, 1);
   uint64_t row;
   memcpy(&row, emu::lds_ptr(a, 8), 8);
   const int par = emu::wave_rendezvous(&row, 8, 0x54523136u);

@@ -614,3 +614,74 @@ def test_guard_pages_do_catch_a_stray_access():
         "print('survived')\n")
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600)
     assert r.returncode == -11 and "survived" not in r.stdout, (r.returncode, r.stdout, r.stderr[-500:])
+
+
+# ---- LDS bank accounting ----------------------------------------------------------------------
+
+def _bank_ratio(stats):
+    """passes taken / passes a conflict-free access takes, per kind of access that occurred"""
+    return {k: v[1] / v[2] for k, v in stats.items() if v[0]}
+
+
+@pytest.mark.parametrize("mode", ["first", "eight_wavefronts", "wavefront_per_head_group", "first_fp8"])
+def test_many_heads_kernels_address_lds_without_bank_conflicts(mode, monkeypatch):
+    """The emulator prices every LDS access the kernels make by address (fragment reads, transposing
+    reads, probability writes) the way the hardware serves it: 16-byte accesses 16 lanes at a time,
+    8-byte ones 32 at a time, 64 banks.  The swizzled tile layouts exist to make these free of
+    conflicts; this is the check that they are, on the code as compiled."""
+    from flagtree_amd import workloads
+    if mode == "first_fp8":
+        cfg, _ = _fp8_cfg(1, 128, 8, 300, pad_frac=0.05)
+    else:
+        cfg = workloads.decode_bf16("cpu", batch=1, heads=128, pages_per_seq=8, topk=300, pad_frac=0.05)
+    if mode in ("eight_wavefronts", "wavefront_per_head_group"):
+        monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1" if mode == "eight_wavefronts" else "2")
+    harness.lds_profile_start()
+    try:
+        out, lse, rc = harness.forward(cfg, n_splits=2)
+    finally:
+        stats = harness.lds_profile_stop()
+    assert rc == 0
+    _check(cfg, out, lse)
+    assert stats["read"][0] > 1000 and stats["read_tr"][0] > 1000, stats
+    assert all(r == 1.0 for r in _bank_ratio(stats).values()), stats
+
+
+def test_few_heads_kernels_transposing_reads_take_two_passes(monkeypatch):
+    """Known and accepted: the few-heads kernels keep rows at a padded stride (1168 bytes), which
+    frees the score reads of conflicts but leaves the P.V transposing reads two-way conflicted (a
+    stride cannot serve both; the many-heads kernels swizzle instead).  Those reads are a few
+    percent of an instruction-bound loop.  The figure is pinned so that a layout change shows up."""
+    from flagtree_amd import workloads
+    for env, cfg in ((None, workloads.decode_bf16("cpu", batch=1, heads=16, pages_per_seq=8, topk=300, pad_frac=0.05)),
+                     (None, _fp8_cfg(1, 16, 8, 300, pad_frac=0.05)[0]),
+                     ("FLAGTREE_SMLA_FEW_FP8", _fp8_cfg(1, 16, 8, 300, pad_frac=0.05)[0])):
+        if env:
+            monkeypatch.setenv(env, "1")
+        harness.lds_profile_start()
+        try:
+            out, lse, rc = harness.forward(cfg, n_splits=2)
+        finally:
+            stats = harness.lds_profile_stop()
+        assert rc == 0 and stats["read_tr"][0] > 100
+        assert _bank_ratio(stats)["read_tr"] == 2.0, stats
+
+
+def test_gemm_kernels_address_lds_without_bank_conflicts():
+    lib = harness.lib()
+    for (m, n, k) in ((512, 512, 128), (384, 256, 128)):          # the 256 x 256 kernel, the 128 x 256 kernel
+        g = torch.Generator().manual_seed(m)
+        x = (torch.randn((m, k), generator=g) * 0.1).to(torch.bfloat16)
+        w = (torch.randn((k, n), generator=g) * 0.1).to(torch.bfloat16)
+        part = torch.randn((m, n), generator=g)
+        out = torch.empty((m, n), dtype=torch.bfloat16)
+        harness.lds_profile_start()
+        try:
+            rc = lib.smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), part.data_ptr(), out.data_ptr(), m, n, k, 1, m * n, None)
+        finally:
+            stats = harness.lds_profile_stop()
+        assert rc == 0
+        want = oracle.gemm_rs_local(to_np(x), to_np(w), to_np(part), 1)
+        assert max_abs(to_np(out).reshape(want.shape), want) <= 1e-2
+        assert stats["read_tr"][0] > 500 and all(r == 1.0 for r in _bank_ratio(stats).values()), stats
+
