@@ -231,6 +231,7 @@ const uint8_t* wave_slot(int parity, int lane) { return g_cur->lane.wave->slot[p
 bool wave_lane_live(int lane) { return g_cur->lane.wave->lane_live[lane]; }
 
 void block_barrier() {
+  g_work.barriers_lane_calls++;
   const unsigned long long my_gen = g_block.gen;
   g_block.arrived++;
   if (g_block.arrived == g_block.live) {
@@ -257,10 +258,17 @@ uint8_t* lds_ptr(uint32_t addr, size_t bytes) {
   return reinterpret_cast<uint8_t*>(__start_emu_lds) + addr;
 }
 
+WorkCounts g_work = {0, 0, 0, 0, 0, 0, 0};
+void count_mfma(int m, int k) {
+  g_work.mfma_lane_calls++;
+  g_work.mfma_flops += 2ull * m * m * k / kWave;          // a lane's share
+}
+
 bool g_lds_profile = false;
 unsigned long long g_lds_stats[9] = {0};
 
 void lds_account(uint32_t addr, int bytes, int kind) {
+  (kind == 2 ? g_work.lds_write_bytes : g_work.lds_read_bytes) += (unsigned long long)bytes;
   if (!g_lds_profile) return;
   const int par = wave_rendezvous(&addr, sizeof(addr), 0x4c424b30u + (uint32_t)kind);
   Lane* me = self();
@@ -302,6 +310,8 @@ void lds_account(uint32_t addr, int bytes, int kind) {
 
 void dma_issue(const void* src, uint32_t lds_dst, int bytes) {
   if (bytes != 0 && bytes != 4 && bytes != 16) fail("dma of %d bytes per lane", bytes);
+  g_work.dma_bytes += (unsigned long long)bytes;
+  g_work.dma_lane_calls += bytes != 0;
   if (g_dma_eager) {
     if (bytes == 0) return;
     memcpy(lds_ptr(lds_dst, bytes), src, bytes);
@@ -389,6 +399,17 @@ void emu_set_cu_count(int n) { emu::g_cu_count = n; }
 void emu_set_lds_profile(int on) {
   emu::g_lds_profile = on != 0;
   for (auto& v : emu::g_lds_stats) v = 0;
+}
+void emu_work_counts(double out[7], int reset) {
+  const emu::WorkCounts& w = emu::g_work;
+  out[0] = (double)w.mfma_lane_calls / emu::kWave;
+  out[1] = (double)w.mfma_flops;
+  out[2] = (double)w.lds_read_bytes;
+  out[3] = (double)w.lds_write_bytes;
+  out[4] = (double)w.dma_bytes;
+  out[5] = (double)w.dma_lane_calls / emu::kWave;
+  out[6] = (double)w.barriers_lane_calls / emu::kWave;
+  if (reset) emu::g_work = emu::WorkCounts{0, 0, 0, 0, 0, 0, 0};
 }
 void emu_lds_profile(unsigned long long out[9]) {
   for (int i = 0; i < 9; ++i) out[i] = emu::g_lds_stats[i];

@@ -60,6 +60,12 @@ void dma_wait(int allowed_in_flight);
 // serves it: 16-byte accesses 16 lanes at a time, 8-byte accesses 32 lanes at a time, 64 banks of
 // 4 bytes, one pass per distinct word a bank is asked for.  kind: 0 read, 1 transposing read, 2 write.
 void lds_account(uint32_t addr, int bytes, int kind);
+// Work counters (always on, cheap): per-lane calls scaled to wavefront instructions by the caller.
+void count_mfma(int m, int k);                        // one lane's share of a wavefront MFMA: M x M x K
+struct WorkCounts {
+  unsigned long long mfma_lane_calls, mfma_flops, lds_read_bytes, lds_write_bytes, dma_bytes, dma_lane_calls, barriers_lane_calls;
+};
+extern WorkCounts g_work;
 
 void launch(Dim3 grid, Dim3 block, const std::function<void()>& body);
 int cu_count();                       // what the stand-in device reports as its number of compute units
@@ -77,4 +83,7 @@ void emu_set_cu_count(int n);            // before the library's first query (it
 void emu_set_lds_profile(int on);        // 1: count bank passes of the kernels' addressed LDS accesses (slower); resets the counts
 // out[3 * kind + 0] wavefront instructions, + 1 passes they took, + 2 passes a conflict-free access would take
 void emu_lds_profile(unsigned long long out[9]);
+// out: MFMA wavefront instructions, MFMA flops, addressed LDS bytes read, written, global -> LDS bytes moved,
+// move wavefront instructions (a partly filled one counts by its active lanes / 64), workgroup barriers x wavefronts
+void emu_work_counts(double out[7], int reset);
 }

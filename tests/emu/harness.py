@@ -35,6 +35,7 @@ def lib():
         l.emu_set_cu_count.argtypes = [ctypes.c_int]
         l.emu_set_lds_profile.argtypes = [ctypes.c_int]
         l.emu_lds_profile.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
+        l.emu_work_counts.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.c_int]
         l.emu_set_cu_count(EMU_CUS)                      # before the library's first (cached) query
         _lib = l
     return _lib
@@ -57,6 +58,16 @@ def lds_profile_stop():
     lib().emu_lds_profile(out)
     lib().emu_set_lds_profile(0)
     return {k: tuple(int(out[3 * i + j]) for j in range(3)) for i, k in enumerate(("read", "read_tr", "write"))}
+
+
+def work_counts(reset=True):
+    """What the emulated kernels have done since the last reset: MFMA wavefront instructions and
+    flops, LDS bytes read / written by address, bytes moved global -> LDS and the wavefront
+    instructions that moved them, workgroup barriers (times wavefronts)."""
+    out = (ctypes.c_double * 7)()
+    lib().emu_work_counts(out, 1 if reset else 0)
+    keys = ("mfma", "mfma_flops", "lds_read_bytes", "lds_write_bytes", "dma_bytes", "dma_instr", "barriers_x_waves")
+    return dict(zip(keys, (float(v) for v in out)))
 
 
 _FORMATS = {"bf16": 0, "fp8_e4m3_b128": 1, "f32": 2}

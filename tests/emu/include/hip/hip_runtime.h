@@ -260,6 +260,7 @@ template <int M, int K, int KPL, int NOUT, typename Frag, typename Acc>
 inline Acc mfma(Frag a, Frag b, Acc c, uint32_t tag) {
   static_assert(sizeof(Frag) == 2 * KPL, "fragment = KPL 16-bit values");
   struct Post { Frag a, b; } post{a, b};
+  count_mfma(M, K);
   const int par = wave_rendezvous(&post, sizeof(post), tag);
   const int l = self()->lane, n = l % M;
   // column n of B once: K values

@@ -685,3 +685,26 @@ def test_gemm_kernels_address_lds_without_bank_conflicts():
         assert max_abs(to_np(out).reshape(want.shape), want) <= 1e-2
         assert stats["read_tr"][0] > 500 and all(r == 1.0 for r in _bank_ratio(stats).values()), stats
 
+
+def test_work_per_unit_of_the_three_many_heads_kernels(monkeypatch):
+    """What each design does per 16 tokens x 128 heads, counted on the code as it runs: the same
+    matrix work, and the LDS and global -> LDS traffic the designs were made to differ in."""
+    from flagtree_amd import workloads
+    cfg = workloads.decode_bf16("cpu", batch=1, heads=128, pages_per_seq=40, topk=1024, pad_frac=0.0)
+    units = 1024 * 128 / (16 * 128)
+    got = {}
+    for name, mode in (("first", None), ("eight_wavefronts", "1"), ("wavefront_per_head_group", "2")):
+        if mode:
+            monkeypatch.setenv("FLAGTREE_SMLA_WIDE", mode)
+        harness.work_counts()
+        out, lse, rc = harness.forward(cfg, n_splits=1)
+        assert rc == 0
+        got[name] = {k: v / units for k, v in harness.work_counts().items()}
+    for w in got.values():
+        assert abs(w["mfma_flops"] - 2 * 16 * 128 * (576 + 512)) < 1.0          # 4.456 MFLOP, nothing computed twice
+    kb = lambda name, key: round(got[name][key] / 1024, 1)       # (the page-table row's move adds a few bytes per unit)
+    assert kb("first", "dma_bytes") == 36.0 and kb("eight_wavefronts", "dma_bytes") == 18.0 and kb("wavefront_per_head_group", "dma_bytes") == 18.0
+    assert kb("first", "lds_read_bytes") == 144.0 and kb("eight_wavefronts", "lds_read_bytes") == 216.0
+    assert kb("wavefront_per_head_group", "lds_read_bytes") == 136.0 and got["wavefront_per_head_group"]["lds_write_bytes"] == 0.0
+    assert got["wavefront_per_head_group"]["barriers_x_waves"] < got["first"]["barriers_x_waves"] < got["eight_wavefronts"]["barriers_x_waves"]
+
