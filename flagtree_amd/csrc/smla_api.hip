@@ -28,8 +28,8 @@ int check_common(const void* q, const void* kv, const int32_t* indices, const vo
 // Kernels that have passed the parity checks but whose speed has not been measured on hardware
 // yet stay behind a switch until it has (read at every call): FLAGTREE_SMLA_FEW_FP8=1 sends few-heads launches over an
 // fp8 cache to the two-workgroups-per-CU kernel (smla_mfma_few_fp8.hip).  Read at every call.
-// FLAGTREE_SMLA_WIDE=1 or 2 sends many-heads launches over a bf16 cache to a 128-heads-per-workgroup
-// kernel: 1 = eight wavefronts (smla_mfma_wide.hip), 2 = a wavefront per 32 heads (smla_mfma_group.hip).
+// FLAGTREE_SMLA_WIDE=1 or 2 sends many-heads launches to a 128-heads-per-workgroup kernel: 1 = eight
+// wavefronts (smla_mfma_wide.hip, bf16 cache only), 2 = a wavefront per 32 heads (smla_mfma_group.hip).
 int wide_mode() {                            // 0: off
   const char* e = getenv("FLAGTREE_SMLA_WIDE");
   return e == nullptr ? 0 : (e[0] == '1' ? 1 : (e[0] == '2' ? 2 : 0));
@@ -124,7 +124,7 @@ int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t t
   // (the opt-in fp8 kernel keeps two workgroups per CU; every further split adds a partial to publish and fold)
   const bool few_fp8 = kv_format == SMLA_KV_FP8_B128 && n_heads <= 32 && few_fp8_enabled();
   const int slots = few_fp8 ? 2 * device_cus() : device_cus();
-  const bool wide = kv_format == SMLA_KV_BF16 && n_heads > 32 && wide_enabled();
+  const bool wide = n_heads > 32 && ((kv_format == SMLA_KV_BF16 && wide_mode() != 0) || (kv_format == SMLA_KV_FP8_B128 && wide_mode() == 2));
   const int per_wg = n_heads <= 32 ? 16 : (wide ? 128 : 64);
   const long long groups = (long long)n_tokens * ((n_heads + per_wg - 1) / per_wg);
   int want = (int)((slots + groups - 1) / groups);
@@ -195,7 +195,8 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
     p.part_out = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + SMLA_WS_COUNTER_BYTES);
     p.part_lse = p.part_out + (size_t)n_tokens * n_splits * n_heads * d_v;
   }
-  if (n_heads > 32 && kv_format == SMLA_KV_BF16 && wide_enabled()) return wide_mode() == 2 ? launch_fwd_group(p, s) : launch_fwd_wide(p, s);
+  if (n_heads > 32 && wide_mode() == 2 && (kv_format == SMLA_KV_BF16 || kv_format == SMLA_KV_FP8_B128)) return launch_fwd_group(kv_format, p, s);
+  if (n_heads > 32 && wide_mode() == 1 && kv_format == SMLA_KV_BF16) return launch_fwd_wide(p, s);
   if (n_heads > 32) return launch_fwd_tall(kv_format, p, s);
   if (kv_format == SMLA_KV_FP8_B128 && few_fp8_enabled()) return launch_fwd_few_fp8(p, s);
   return launch_fwd_short(kv_format, p, s);

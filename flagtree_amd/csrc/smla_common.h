@@ -45,9 +45,11 @@ struct LogitCap {
   float a, b;                   // a = 2 log2(e) sm_scale / cap,  b = log2(e) cap
   __device__ __forceinline__ LogitCap(float sm_scale, float cap)
       : a(2.f * 1.4426950408889634f * sm_scale / cap), b(1.4426950408889634f * cap) {}
+  // (each instruction takes one of the two constants, so both can stay in scalar registers: a
+  // vector instruction reads at most one scalar register)
   __device__ __forceinline__ float operator()(float raw) const {
     const float e = __builtin_amdgcn_exp2f(raw * a);
-    return __builtin_fmaf(-2.f * b, __builtin_amdgcn_rcpf(e + 1.f), b);
+    return b * __builtin_fmaf(-2.f, __builtin_amdgcn_rcpf(e + 1.f), 1.f);
   }
 };
 
@@ -200,7 +202,7 @@ int launch_fwd_scalar(int kv_format, const Params& p, hipStream_t s);
 int launch_fwd_tall(int kv_format, const Params& p, hipStream_t s);    // n_heads > 32 (logit cap: a second instantiation)
 int launch_fwd_short(int kv_format, const Params& p, hipStream_t s);   // n_heads <= 32
 int launch_fwd_wide(const Params& p, hipStream_t s);                   // n_heads > 32, bf16 rows, 128 heads per workgroup, 8 wavefronts (opt-in)
-int launch_fwd_group(const Params& p, hipStream_t s);                  // n_heads > 32, bf16 rows, 128 heads per workgroup, a wavefront per 32 heads (opt-in)
+int launch_fwd_group(int kv_format, const Params& p, hipStream_t s);   // n_heads > 32, bf16 rows or fp8 records, 128 heads per workgroup, a wavefront per 32 heads (opt-in)
 int launch_fwd_few_fp8(const Params& p, hipStream_t s);                // n_heads <= 32, fp8 records, two workgroups per CU (opt-in)
 int launch_merge(const float* part_out, const float* part_lse, void* out, float* lse,
                  int n_tokens, int n_heads, int d_v, int n_splits, hipStream_t s);

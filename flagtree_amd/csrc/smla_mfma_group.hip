@@ -27,6 +27,7 @@
 //   ds_read_b64_tr_b16: inside each group of 16 lanes, lane i receives element (i%4) of the
 //   8-byte rows addressed by lanes (i/4), (i/4)+4, (i/4)+8, (i/4)+12.
 #include "smla_common.h"
+#include "smla_fp8_pipe.h"
 
 namespace smla {
 namespace {
@@ -69,10 +70,20 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-__device__ __forceinline__ uint32_t rope_slot(int r, int c) {     // byte offset of RoPE chunk c of tile row r in the tile
+__device__ __forceinline__ uint32_t rope_slot(int r, int c) {     // byte offset of RoPE chunk c of tile row r in a tile's RoPE block
   const int p = r >> 1;
-  return kRopeBase + p * 256 + ((((r & 1) << 3) | (c ^ (p & 7))) << 4);
+  return p * 256 + ((((r & 1) << 3) | (c ^ (p & 7))) << 4);
 }
+
+// fp8 records: raw records -> LDS by moves, LDS -> LDS conversion (smla_fp8_pipe.h).  This kernel's
+// row xor: swz(row0 + 2k) = swz(row0) ^ 4k for row0 = 8 * wave + l/32 (bits 1-3 count the row within its eight).
+struct GroupLayout {
+  __device__ static constexpr int swz(int r) { return ((r & 7) << 1) | ((r >> 3) & 1); }
+  __device__ static constexpr int store_xor(int k) { return 4 * k; }
+};
+using Fp8Pipe = fp8pipe::Pipe;
+using Fp8Convert = fp8pipe::Convert<GroupLayout>;
+static_assert(fp8pipe::kTN == kTN && fp8pipe::kMainStride == kMainStride && fp8pipe::kRopeBase == kRopeBase, "tile geometry");
 
 // A tile's rows go global -> LDS directly: one move brings the first 1 KB of a row (scalar row base
 // + per-lane chunk offset; lane l fetches chunk l ^ swz(row) so the row lands swizzled), one more
@@ -112,28 +123,28 @@ __device__ __forceinline__ void wait_dma(int younger_tiles) {
   else hw::wait_vmcnt<0>();
 }
 
-// Raw scores of a tile: sa[2 * tt + ht] = S^T of token half tt (tile rows 16 tt .. + 15) against
+// Raw scores of a tile (body at `tile`, RoPE block at `rope`): sa[2 * tt + ht] = S^T of token half tt (tile rows 16 tt .. + 15) against
 // head tile ht (heads 16 ht .. + 15 of the group).  Four independent accumulation chains; a K
 // fragment feeds two MFMAs.  `side(ks)` is called once per k-step.
-template <typename Side>
-__device__ __forceinline__ void tile_scores(uint32_t tile, const bf16x8 (&qf)[kDqk / 32][2], f32x4 (&sa)[4], int lane, Side side) {
+template <int kAhead = kPrefetchA, typename Side>
+__device__ __forceinline__ void tile_scores(uint32_t tile, uint32_t rope, const bf16x8 (&qf)[kDqk / 32][2], f32x4 (&sa)[4], int lane, Side side) {
   constexpr int kSteps = kDqk / 32, kMainSteps = kDv / 32;
   const int l16 = lane & 15, q4 = lane >> 4;
   // row 16 tt + l16: swz depends on l16 only; chunk 4 ks + q4 sits at ((4 ks + q4) ^ swz) * 16
   const uint32_t kmain = tile + l16 * kMainStride + ((q4 ^ swz(l16)) << 4);
   auto frag = [&](int ks, int tt) {
     if (ks < kMainSteps) return hw::lds_read_b128((kmain ^ (uint32_t)((ks & 3) << 6)) + (ks >> 2) * 256 + tt * 16 * kMainStride);
-    return hw::lds_read_b128(tile + rope_slot(16 * tt + l16, 4 * (ks - kMainSteps) + q4));
+    return hw::lds_read_b128(rope + rope_slot(16 * tt + l16, 4 * (ks - kMainSteps) + q4));
   };
 #pragma unroll
   for (int i = 0; i < 4; ++i) sa[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   __builtin_amdgcn_sched_barrier(0);
   bf16x8 a[kSteps][2];
 #pragma unroll
-  for (int ks = 0; ks < kPrefetchA; ++ks) { a[ks][0] = frag(ks, 0); a[ks][1] = frag(ks, 1); }
+  for (int ks = 0; ks < kAhead; ++ks) { a[ks][0] = frag(ks, 0); a[ks][1] = frag(ks, 1); }
 #pragma unroll
   for (int ks = 0; ks < kSteps; ++ks) {
-    if (ks + kPrefetchA < kSteps) { a[ks + kPrefetchA][0] = frag(ks + kPrefetchA, 0); a[ks + kPrefetchA][1] = frag(ks + kPrefetchA, 1); }
+    if (ks + kAhead < kSteps) { a[ks + kAhead][0] = frag(ks + kAhead, 0); a[ks + kAhead][1] = frag(ks + kAhead, 1); }
     sa[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ks][0], qf[ks][0], sa[0], 0, 0, 0);
     sa[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ks][0], qf[ks][1], sa[1], 0, 0, 0);
     sa[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ks][1], qf[ks][0], sa[2], 0, 0, 0);
@@ -141,10 +152,10 @@ __device__ __forceinline__ void tile_scores(uint32_t tile, const bf16x8 (&qf)[kD
     side(ks);
   }
 #pragma unroll
-  for (int ks = 0; ks < kPrefetchA; ++ks) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // DS read
+  for (int ks = 0; ks < kAhead; ++ks) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // DS read
 #pragma unroll
   for (int ks = 0; ks < kSteps; ++ks) {
-    if (ks + kPrefetchA < kSteps) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    if (ks + kAhead < kSteps) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);                                         // MFMA
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -157,12 +168,16 @@ __device__ __forceinline__ void tile_scores(uint32_t tile, const bf16x8 (&qf)[kD
 // 16 ct + 4 (p%4) .. + 3 of token 4q + p/4 (first read: k-slots 8q .. 8q+3) and of token
 // 16 + 4q + p/4 (second read: k-slots 8q+4 .. 8q+7).
 // `valu(i)` is independent vector work of the caller, pinned behind MFMA pair i.
-template <bool kPinValu, typename Valu>
+// kFreshAddr: the lane's part of the addresses is worked out afresh in every call (the variant short
+// of registers cannot afford the eight xor-ed copies the compiler would otherwise keep for the whole kernel).
+template <bool kPinValu, bool kFreshAddr, int kAhead = kPrefetchB, typename Valu>
 __device__ __forceinline__ void tile_accumulate(uint32_t tile, const bf16x8 (&pa)[2], f32x4 (&acc)[2][kColTiles], int lane, Valu valu) {
   const int q4 = lane >> 4, p16 = lane & 15;
   const int row = 4 * q4 + (p16 >> 2);                           // token of the first read; the second read's is row + 16 (same swz)
   // columns 16 ct + 4 (p%4): chunk 2 ct + (p%4 >> 1), byte 8 (p%4 & 1); the chunk moves to (2 ct) ^ swz(row) ^ (p%4 >> 1)
-  const uint32_t vbase = tile + row * kMainStride + ((swz(row) ^ ((p16 & 3) >> 1)) << 4) + 8 * (p16 & 1);
+  uint32_t lane_part = row * kMainStride + ((swz(row) ^ ((p16 & 3) >> 1)) << 4) + 8 * (p16 & 1);
+  if constexpr (kFreshAddr) hw::pin(lane_part);
+  const uint32_t vbase = tile + lane_part;
   __builtin_amdgcn_sched_barrier(0);
   bf16x4 lo[kColTiles], hi[kColTiles];
   // chunk 2 ct: the xor with swz touches its low four bits only, so column tiles 8 apart share an
@@ -173,10 +188,10 @@ __device__ __forceinline__ void tile_accumulate(uint32_t tile, const bf16x8 (&pa
     hi[ct] = hw::lds_read_tr16_b64(a + 16 * kMainStride);
   };
 #pragma unroll
-  for (int ct = 0; ct < kPrefetchB; ++ct) load(ct);
+  for (int ct = 0; ct < kAhead; ++ct) load(ct);
 #pragma unroll
   for (int ct = 0; ct < kColTiles; ++ct) {
-    if (ct + kPrefetchB < kColTiles) load(ct + kPrefetchB);
+    if (ct + kAhead < kColTiles) load(ct + kAhead);
     const bf16x8 bv = __builtin_shufflevector(lo[ct], hi[ct], 0, 1, 2, 3, 4, 5, 6, 7);
     acc[0][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[0], bv, acc[0][ct], 0, 0, 0);
     acc[1][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[1], bv, acc[1][ct], 0, 0, 0);
@@ -188,18 +203,21 @@ __device__ __forceinline__ void tile_accumulate(uint32_t tile, const bf16x8 (&pa
   }
   if constexpr (!kPinValu) {
 #pragma unroll
-    for (int ct = 0; ct < kPrefetchB; ++ct) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    for (int ct = 0; ct < kAhead; ++ct) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ++ct) {
-      if (ct + kPrefetchB < kColTiles) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      if (ct + kAhead < kColTiles) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
     }
   }
   __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool CAP>
+template <int FMT, bool CAP>
 __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks) {
+  // the ring area: bf16 has four whole tiles (body + RoPE block each); fp8 see smla_fp8_pipe.h
+  constexpr bool kFp8 = FMT == SMLA_KV_FP8_B128;
+  static_assert(Fp8Pipe::kRingBytes <= kSlots * kTileBytes, "the fp8 carving fits the same area");
   __shared__ __attribute__((aligned(1024))) uint8_t s_ring[kSlots * kTileBytes];   // swizzle xors need 1 KB alignment
   __shared__ int32_t s_rows[kChunk];
   __shared__ float s_inv[4][32];                                  // per-head normalisers (epilogue)
@@ -237,13 +255,14 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
       rr[k] = j < c1 ? (listed ? v : (j < v ? j : -1)) : -1;
     }
   };
-  // the sequence's page-table row goes global -> LDS (last ring slot, free until the first chunk's
+  // the sequence's page-table row goes global -> LDS (last tile body, free until the first chunk's
   // row list exists), issued ahead of the index loads so that it has landed once they have
   const int32_t* bt_row = p.block_table ? p.block_table + (size_t)seq * p.bt_stride : nullptr;
   const bool bt_in_lds = bt_row != nullptr && p.bt_stride <= kBtLdsMax && (p.bt_stride & 3) == 0 &&
                          ((uintptr_t)bt_row & 15) == 0;
   const uint32_t lds_tile = hw::lds_addr(&s_ring[0]);
-  const uint32_t lds_bt = lds_tile + (kSlots - 1) * kTileBytes;
+  constexpr int kBtStage = kFp8 ? (Fp8Pipe::kBodies - 1) * kRopeBase : (kSlots - 1) * kTileBytes;
+  const uint32_t lds_bt = lds_tile + kBtStage;
   if (bt_in_lds) {
     for (int c = wave; 256 * c < p.bt_stride; c += 4) {            // 1 KB (256 entries) per instruction
       const int e = 256 * c + 4 * lane;
@@ -269,7 +288,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   if (bt_in_lds) {
     hw::wait_for_loads_of(rr_first[0], rr_first[1], rr_first[2], rr_first[3]);
     __syncthreads();
-    const int32_t* bt_s = reinterpret_cast<const int32_t*>(&s_ring[(kSlots - 1) * kTileBytes]);
+    const int32_t* bt_s = reinterpret_cast<const int32_t*>(&s_ring[kBtStage]);
 #pragma unroll
     for (int k = 0; k < 4; ++k) rr_first[k] = translate_index(p, rr_first[k], bt_s);
   } else {
@@ -328,12 +347,40 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
       const int n_tiles = (n_valid + kTN - 1) / kTN;
       if (n_tiles == 0) continue;
 
+      // bf16: tile `it` lives in ring slot it % kSlots.  fp8: its body in body it % 3, its RoPE block in
+      // block it % 3, its raw records in raw block it % 2.
+      [[maybe_unused]] Fp8Pipe pipe;
+      [[maybe_unused]] Fp8Convert cv;
       DmaTile dma;
-      auto tile_addr = [&](int it) { return lds_tile + (it & (kSlots - 1)) * kTileBytes; };
+      uint32_t ring = lds_tile;
+      if constexpr (kFp8) hw::pin_uniform(ring);   // (per-lane addresses of the first tiles are worked out per chunk, not held from the top)
+      auto tile_addr = [&](int it) {
+        if constexpr (kFp8) return ring + (uint32_t)(it % Fp8Pipe::kBodies) * kRopeBase;
+        else return ring + (it & (kSlots - 1)) * kTileBytes;
+      };
+      auto rope_addr = [&](int it) {
+        if constexpr (kFp8) return ring + Fp8Pipe::kRopeRing + (uint32_t)(it % Fp8Pipe::kRopes) * fp8pipe::kRopeBlock;
+        else return ring + (it & (kSlots - 1)) * kTileBytes + kRopeBase;
+      };
+      [[maybe_unused]] auto pipe_begin = [&](int it, int ln) {
+        pipe.begin(kv, s_rows, it * kTN, n_valid,
+                   ring + Fp8Pipe::kRawRing + (it & 1) * Fp8Pipe::kRawSlot + wave * Fp8Pipe::kRawWave, rope_addr(it), wave, ln);
+      };
+      [[maybe_unused]] auto convert_begin = [&](int it, int ln) {
+        cv.raw = &s_ring[Fp8Pipe::kRawRing + (it & 1) * Fp8Pipe::kRawSlot + wave * Fp8Pipe::kRawWave];
+        cv.body = &s_ring[(it % Fp8Pipe::kBodies) * kRopeBase];
+        cv.wave = wave; cv.lane = ln;
+      };
       auto fetch_whole = [&](int it) {
-        dma.begin(kv, s_rows, it * kTN, n_valid, tile_addr(it), wave, lane);
+        if constexpr (!kFp8) {
+          dma.begin(kv, s_rows, it * kTN, n_valid, tile_addr(it), wave, lane);
 #pragma unroll
-        for (int j = 0; j < kDmaSteps; ++j) dma.step(j);
+          for (int j = 0; j < kDmaSteps; ++j) dma.step(j);
+        } else {
+          pipe_begin(it, lane);
+#pragma unroll
+          for (int j = 0; j < Fp8Pipe::kSteps; ++j) pipe.step(j);
+        }
       };
       // scores of tile `it` -> the lane's probabilities as the A operands of the P.V MFMAs (not pipelined:
       // first tile and tail).  s[tt][ht][r]: token 16 tt + 4 q4 + r, head 16 ht + l16.
@@ -388,18 +435,34 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
       // issue order, so waiting for the moves also waits for everything older), tile 2 rides on
       // the scores of tile 0
       for (int it = 0; it < min(n_tiles, 2); ++it) fetch_whole(it);
-      wait_dma(n_tiles > 1 ? 1 : 0);
+      if constexpr (!kFp8) {
+        wait_dma(n_tiles > 1 ? 1 : 0);
+      } else {
+        // fp8: convert tile 0, send for tile 2 (its raw block is free again), convert tile 1
+        // (a wavefront's lanes read scale chunks that other lanes of it fetched: wave_lds_order)
+        if (n_tiles > 1) hw::wait_vmcnt<Fp8Pipe::kSteps>(); else hw::wait_vmcnt<0>();
+        hw::wave_lds_order();
+        convert_begin(0, lane);
+        cv.whole_tile();
+        if (n_tiles > 2) fetch_whole(2);
+        if (n_tiles > 1) {
+          if (n_tiles > 2) hw::wait_vmcnt<Fp8Pipe::kSteps>(); else hw::wait_vmcnt<0>();
+          hw::wave_lds_order();
+          convert_begin(1, lane);
+          cv.whole_tile();
+        }
+      }
 #pragma unroll
       for (int ks = 0; ks < kDqk / 32; ++ks) hw::wait_for_loads_of(qf[ks][0], qf[ks][1]);   // (tells the compiler that Q is there)
       __syncthreads();                       // tile 0 landed
       bf16x8 pa[2];                          // probabilities of the tile to be accumulated next
       {
         f32x4 sa[4];
-        if (n_tiles > 2) {
+        if (!kFp8 && n_tiles > 2) {
           dma.begin(kv, s_rows, 2 * kTN, n_valid, tile_addr(2), wave, lane);
-          tile_scores(tile_addr(0), qf, sa, lane, [&](int ks) { if ((ks & 1) == 0) dma.step(ks >> 1); });
+          tile_scores(tile_addr(0), rope_addr(0), qf, sa, lane, [&](int ks) { if ((ks & 1) == 0) dma.step(ks >> 1); });
         } else {
-          tile_scores(tile_addr(0), qf, sa, lane, [](int) {});
+          tile_scores(tile_addr(0), rope_addr(0), qf, sa, lane, [](int) {});
         }
         finish_scores(0, sa, pa);
       }
@@ -410,15 +473,40 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
       const int n_main = max(n_tiles - (kSlots - 1), 0);
       int it = 0;
       for (; it < n_main; ++it) {
-        wait_dma(1);                         // tile it+1 was issued two iterations ago; only tile it+2 is still outstanding
-        __syncthreads();                     // tile it+1 landed for everyone, tile it-1 is consumed by everyone
-        dma.begin(kv, s_rows, (it + kSlots - 1) * kTN, n_valid, tile_addr(it + kSlots - 1), wave, lane);
+        if constexpr (!kFp8) wait_dma(1);    // tile it+1 was issued two iterations ago; only tile it+2 is still outstanding
+        __syncthreads();                     // tile it+1 landed / converted for everyone, tile it-1 is consumed by everyone
+        if constexpr (!kFp8) {
+          dma.begin(kv, s_rows, (it + kSlots - 1) * kTN, n_valid, tile_addr(it + kSlots - 1), wave, lane);
+        }
+        // fp8: the lane id is taken afresh in every iteration, so that the dozen per-lane address parts
+        // derived from it are worked out here (a few instructions each) rather than held in registers
+        // for the whole kernel, which this variant cannot afford
+        int ln = lane;
+        if constexpr (kFp8) {
+          hw::pin(ln);
+          pipe_begin(it + 3, ln);            // send for tile it+3; the raw records of tile it+2 are converted under the P.V MFMAs below
+          convert_begin(it + 2, ln);
+        }
         f32x4 sa[4];
-        tile_scores(tile_addr(it + 1), qf, sa, lane, [&](int ks) { if ((ks & 1) == 0) dma.step(ks >> 1); });
+        // (fp8: the conversion shares the loop's registers: one fragment pair and one column tile less ahead)
+        tile_scores<kFp8 ? kPrefetchA - 1 : kPrefetchA>(tile_addr(it + 1), rope_addr(it + 1), qf, sa, ln, [&](int ks) {
+          if ((ks & 1) == 0) {
+            if constexpr (!kFp8) dma.step(ks >> 1);
+            else if ((ks >> 1) < Fp8Pipe::kSteps) pipe.step(ks >> 1);
+          }
+        });
         float pr[8];
         hw::u32x4 pw[2];
         bool over = false;
-        tile_accumulate<true>(tile_addr(it), pa, acc, lane, [&](int i) {
+        tile_accumulate<true, kFp8, kFp8 ? kPrefetchB - 1 : kPrefetchB>(tile_addr(it), pa, acc, ln, [&](int i) {
+          if constexpr (kFp8) {
+            // slices 23..27 carry the conversion, after the softmax (slices 0..22) has given its
+            // registers back: the read of chunk 0, then per chunk its two halves, its stores and the
+            // next chunk's read.  The moves of tile it+3, just issued, stay in flight; everything
+            // older has landed after the wait.
+            if (i == 23) { hw::wait_vmcnt<Fp8Pipe::kSteps>(); hw::wave_lds_order(); cv.load(0); }
+            else if (i >= 24 && i < 28) { cv.half(0); cv.half(1); cv.store(i - 24); if (i < 27) cv.load(i - 23); }
+          }
           if (i < 4) {                       // slices 0..3: one score block each: cap, per-lane maximum, overflow test
             if constexpr (CAP) {
 #pragma unroll
@@ -449,15 +537,23 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
       // ---- tail: the last tiles, nothing left to fetch
       for (; it < n_tiles; ++it) {
         const bool next = it + 1 < n_tiles;
-        if (next) wait_dma(it + 2 < n_tiles ? 1 : 0);
+        if constexpr (!kFp8) { if (next) wait_dma(it + 2 < n_tiles ? 1 : 0); }
         __syncthreads();
+        if constexpr (kFp8) {                // tile it+2 may still await its conversion
+          if (it + 2 < n_tiles) {
+            hw::wait_vmcnt<0>();
+            hw::wave_lds_order();
+            convert_begin(it + 2, lane);
+            cv.whole_tile();
+          }
+        }
         bf16x8 pn[2] = {pa[0], pa[1]};
         if (next) {
           f32x4 sa[4];
-          tile_scores(tile_addr(it + 1), qf, sa, lane, [](int) {});
+          tile_scores(tile_addr(it + 1), rope_addr(it + 1), qf, sa, lane, [](int) {});
           finish_scores(it + 1, sa, pn);
         }
-        tile_accumulate<false>(tile_addr(it), pa, acc, lane, [](int) {});
+        tile_accumulate<false, kFp8>(tile_addr(it), pa, acc, lane, [](int) {});
         pa[0] = pn[0]; pa[1] = pn[1];
       }
     }
@@ -667,19 +763,22 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   if (wave == 0 && lane_e == 0) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
 }
 
-template <bool CAP>
+template <int FMT, bool CAP>
 int launch_impl(const Params& p, hipStream_t s) {
   const int n_hblocks = (p.n_heads + 127) / 128;
   const long long blocks = ((long long)p.n_tokens + 7) / 8 * 8 * n_hblocks * p.n_splits;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
-  hipLaunchKernelGGL(fwd_group_kernel<CAP>, dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_group_kernel<FMT, CAP>), dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
   return hip_status(hipGetLastError());
 }
 
 }  // namespace
 
-int launch_fwd_group(const Params& p, hipStream_t s) {
-  return p.logit_cap > 0.f ? launch_impl<true>(p, s) : launch_impl<false>(p, s);
+int launch_fwd_group(int kv_format, const Params& p, hipStream_t s) {
+  const bool cap = p.logit_cap > 0.f;
+  if (kv_format == SMLA_KV_BF16) return cap ? launch_impl<SMLA_KV_BF16, true>(p, s) : launch_impl<SMLA_KV_BF16, false>(p, s);
+  if (kv_format == SMLA_KV_FP8_B128) return cap ? launch_impl<SMLA_KV_FP8_B128, true>(p, s) : launch_impl<SMLA_KV_FP8_B128, false>(p, s);
+  return SMLA_EINVAL_SHAPE;
 }
 
 }  // namespace smla

@@ -27,6 +27,7 @@
 //   ds_read_b64_tr_b16: inside each group of 16 lanes, lane i receives element (i%4) of the
 //   8-byte rows addressed by lanes (i/4), (i/4)+4, (i/4)+8, (i/4)+12.
 #include "smla_common.h"
+#include "smla_fp8_pipe.h"
 
 namespace smla {
 
@@ -119,92 +120,15 @@ __device__ __forceinline__ uint32_t rope_slot(int r, int c) {     // byte offset
   return p * 256 + ((((r & 1) << 3) | (c ^ (p & 7))) << 4);
 }
 
-// fp8 records (512 e4m3 values, 4 float scales, 64 bf16 RoPE values = 656 bytes) reach LDS raw,
-// by the same global -> LDS moves, and are dequantised from LDS to LDS: no register waits for
-// memory.  Wavefront w owns tile rows 8w .. 8w+7 from end to end.  Move j = 0..3 fetches the value
-// chunks of its rows 2j and 2j+1 (lane l: row 2j + l/32, chunk l%32) into 1 KB of its raw block,
-// move 4 the eight scale chunks (lanes 0..7, one row each) into the 128 bytes behind them, move 5
-// the RoPE parts straight into the tile's RoPE block (they are bf16 already).  Later every lane
-// turns the four value chunks it fetched itself (raw block byte 16*l + 1024*k) into
-// bf16(float(e4m3) * scale) in the tile body.  Only the wavefront's own moves feed its
-// conversion, so a wait on its own counter is all the synchronisation the raw data needs, and a
-// raw block can be refilled as soon as it is converted.
-// LDS: three tile bodies (one being multiplied, one being scored, one being written), three RoPE
-// blocks (scored, landed, in flight) and two raw blocks per wavefront (converting, in flight).
-struct Fp8Pipe {
-  static constexpr int kRawWave = 8 * (kFp8ScaleOff + 16);     // 4224 bytes: a wavefront's 8 rows, values then scales
-  static constexpr int kRawScales = 8 * kFp8ScaleOff;          // 4096: where the scale chunks start
-  static constexpr int kRawSlot = 4 * kRawWave;                // 16896
-  static constexpr int kSteps = 6;                             // move instructions per wavefront per tile
-  static constexpr int kBodies = 3, kRopes = 3, kRaws = 2;
-  static constexpr int kRopeRing = kBodies * kRopeBase;        // byte offsets in the ring area
-  static constexpr int kRawRing = kRopeRing + kRopes * (kTN * 128);
-  static constexpr int kRingBytes = kRawRing + kRaws * kRawSlot;      // 144384
-  const uint8_t* kv;
-  uint32_t raw_lds, rope_lds;
-  int32_t rid;
-  int wave, lane;
-  // raw_lds_: this wavefront's raw block, rope_lds_: the tile's RoPE block
-  __device__ __forceinline__ void begin(const uint8_t* kv_, const int32_t* rows, int e0, int n_valid,
-                                        uint32_t raw_lds_, uint32_t rope_lds_, int wave_, int lane_) {
-    kv = kv_; raw_lds = raw_lds_; rope_lds = rope_lds_; wave = wave_; lane = lane_;
-    rid = rows[min(e0 + (lane & 31), n_valid - 1)];               // lane l holds the row id of tile row l % 32
-  }
-  __device__ __forceinline__ void step(int j) const {
-    if (j < 4) {
-      const int32_t trow = __shfl(rid, 8 * wave + 2 * j + (lane >> 5));
-      hw::dma_b128(kv + (size_t)trow * kRowBytesFp8 + (lane & 31) * 16, raw_lds + 1024 * j);
-    } else if (j == 4) {
-      const int32_t trow = __shfl(rid, 8 * wave + (lane & 7));
-      hw::dma_b128_first_lanes<8>(kv + (size_t)trow * kRowBytesFp8 + kFp8ScaleOff, raw_lds + kRawScales);
-    } else {
-      const int pair = 4 * wave + (lane >> 4);
-      const int r = 2 * pair + ((lane >> 3) & 1), c = (lane & 7) ^ (pair & 7);
-      const int32_t trow = __shfl(rid, r);
-      hw::dma_b128(kv + (size_t)trow * kRowBytesFp8 + kFp8ScaleOff + 16 + c * 16, rope_lds + wave * 1024);
-    }
-  }
+// fp8 records: raw records -> LDS by moves, LDS -> LDS conversion (smla_fp8_pipe.h).  This kernel's
+// row xor: swz(row0 + 2k) = swz(row0) ^ (8 * (k & 1) | (k >> 1)) for row0 = 8 * wave + l/32.
+struct TallLayout {
+  __device__ static constexpr int swz(int r) { return smla::swz(r); }
+  __device__ static constexpr int store_xor(int k) { return (8 * (k & 1)) | (k >> 1); }
 };
-
-// The conversion of one tile is 4 chunks of 16 values per lane: chunk k is column chunk l % 32 of
-// the wavefront's row l/32 + 2k.  load / half / store are separate so that a caller can thread
-// them through an MFMA stream.
-struct Fp8Convert {
-  uint4 v;
-  float sc;
-  uint32_t o[8];
-  const uint8_t* raw;      // this wavefront's raw block
-  uint8_t* body;           // the tile body being written
-  int wave, lane;
-  __device__ __forceinline__ void load(int k) {
-    v = *reinterpret_cast<const uint4*>(raw + 16 * lane + 1024 * k);
-    sc = *reinterpret_cast<const float*>(raw + Fp8Pipe::kRawScales + 16 * (lane >> 5) + 4 * ((lane & 31) >> 3) + 32 * k);
-  }
-  __device__ __forceinline__ void half(int h) {
-    const uint32_t w[2] = {h == 0 ? v.x : v.z, h == 0 ? v.y : v.w};
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[k], false);
-      const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[k], true);
-      o[4 * h + 2 * k] = pack_bf16(lo[0] * sc, lo[1] * sc);
-      o[4 * h + 2 * k + 1] = pack_bf16(hi[0] * sc, hi[1] * sc);
-    }
-  }
-  __device__ __forceinline__ void store(int k) {
-    // tile row 8*wave + l/32 + 2k, chunks 2*col and 2*col + 1.  With row0 the row of k = 0:
-    // swz(row) = swz(row0) ^ (8 * (k & 1) | (k >> 1)), so one per-lane offset serves all four chunks.
-    const int row0 = 8 * wave + (lane >> 5), col = lane & 31;
-    int off = row0 * kMainStride + (((2 * col) ^ swz(row0)) << 4);
-    hw::pin(off);                                                  // (worked out here, not kept in four registers from the top of the kernel)
-    off = (off ^ (((8 * (k & 1)) | (k >> 1)) << 4)) + 2 * k * kMainStride;
-    *reinterpret_cast<uint4*>(body + off) = make_uint4(o[0], o[1], o[2], o[3]);
-    *reinterpret_cast<uint4*>(body + (off ^ 16)) = make_uint4(o[4], o[5], o[6], o[7]);
-  }
-  __device__ __forceinline__ void whole_tile() {     // (one chunk at a time: where this is called, registers are scarce)
-#pragma unroll 1
-    for (int k = 0; k < 4; ++k) { load(k); half(0); half(1); store(k); }
-  }
-};
+using Fp8Pipe = fp8pipe::Pipe;
+using Fp8Convert = fp8pipe::Convert<TallLayout>;
+static_assert(fp8pipe::kTN == kTN && fp8pipe::kMainStride == kMainStride && fp8pipe::kRopeBase == kRopeBase, "tile geometry");
 
 // ---- per-tile math -------------------------------------------------------------------------
 // Softmax reference handling.  The fast pass takes each head's maximum over the first tile as

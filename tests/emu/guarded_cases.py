@@ -134,6 +134,8 @@ CASES = {
     # 65 heads: the second head group of the second block lies wholly past the last head
     "tall_bf16_empty_head_group_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=65, pages_per_seq=5, topk=200, pad_frac=0.06), 3),
     "tall_fp8_split": forward_case(lambda: fp8_cfg(2, 128, 4, 150), 2),
+    "group_fp8_split": forward_case(lambda: fp8_cfg(2, 128, 4, 150), 2, env={"FLAGTREE_SMLA_WIDE": "2"}),
+    "group_fp8_short_lists": forward_case(lambda: fp8_cfg(3, 65, 2, 40), 1, env={"FLAGTREE_SMLA_WIDE": "2"}),
     "tall_fp8_short_lists": forward_case(lambda: fp8_cfg(3, 65, 2, 40), 1),
     "short_bf16_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=2, heads=16, pages_per_seq=5, topk=200, pad_frac=0.06), 2),
     "short_bf16_ragged_heads": forward_case(lambda: workloads.decode_bf16("cpu", batch=1, heads=9, pages_per_seq=5, topk=150, pad_frac=0.06), 1),

@@ -116,7 +116,27 @@ def test_many_heads_fp8_pipeline_at_every_tile_count(topk, n_splits):
     _check(cfg, out, lse)
 
 
-def test_many_heads_fp8_redo_passes():
+@pytest.mark.parametrize("topk,n_splits,heads", [(1, 1, 40), (33, 1, 128), (64, 2, 65), (97, 1, 128), (128, 1, 96), (129, 2, 128),
+                                                 (200, 3, 128), (1030, 1, 40), (2100, 2, 128)])
+def test_head_group_kernel_fp8_pipeline(topk, n_splits, heads, monkeypatch):
+    """The same raw-record pipeline inside the wavefront-per-head-group kernel (its own row xor)."""
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "2")
+    cfg, _ = _fp8_cfg(1, heads, 40, topk, pad_frac=0.0 if topk < 40 else 0.04)
+    out, lse = _forward_all_ways(cfg, n_splits)
+    _check(cfg, out, lse)
+    os.environ.pop("FLAGTREE_SMLA_WIDE")
+    out1, lse1, rc = harness.forward(cfg, n_splits=n_splits)             # the first kernel
+    assert rc == 0 and max_abs(to_np(out1), to_np(out)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse)) <= 1e-5
+
+
+@pytest.mark.parametrize("mode", ["first", "wavefront_per_head_group"])
+def test_many_heads_fp8_redo_passes(mode, monkeypatch):
+    if mode != "first":
+        monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "2")
+    _many_heads_fp8_redo_passes()
+
+
+def _many_heads_fp8_redo_passes():
     """Scores that outgrow the first tile's reference: the fp8 pipeline runs three times over the list."""
     g = torch.Generator().manual_seed(11)
     latent = (torch.randn((400, 576), generator=g) * 4.0).to(torch.bfloat16)
@@ -408,8 +428,8 @@ def test_random_shapes_against_oracle(seed, few_fp8, monkeypatch):
     paged = rng.random() < 0.7
     ctx = int(rng.choice([64, 300, 1200]))
     if few_fp8 in ("wide", "wide_k"):
-        if fmt != "bf16" or heads <= 32:
-            pytest.skip("the opt-in kernel covers many heads over a bf16 cache")
+        if heads <= 32 or (fmt != "bf16" and few_fp8 == "wide"):
+            pytest.skip("the opt-in kernels cover many heads (the eight-wavefront one over a bf16 cache only)")
         monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1" if few_fp8 == "wide" else "2")
     elif few_fp8:
         if fmt != "fp8_e4m3_b128" or heads > 32:
@@ -623,18 +643,18 @@ def _bank_ratio(stats):
     return {k: v[1] / v[2] for k, v in stats.items() if v[0]}
 
 
-@pytest.mark.parametrize("mode", ["first", "eight_wavefronts", "wavefront_per_head_group", "first_fp8"])
+@pytest.mark.parametrize("mode", ["first", "eight_wavefronts", "wavefront_per_head_group", "first_fp8", "wavefront_per_head_group_fp8"])
 def test_many_heads_kernels_address_lds_without_bank_conflicts(mode, monkeypatch):
     """The emulator prices every LDS access the kernels make by address (fragment reads, transposing
     reads, probability writes) the way the hardware serves it: 16-byte accesses 16 lanes at a time,
     8-byte ones 32 at a time, 64 banks.  The swizzled tile layouts exist to make these free of
     conflicts; this is the check that they are, on the code as compiled."""
     from flagtree_amd import workloads
-    if mode == "first_fp8":
+    if mode.endswith("_fp8"):
         cfg, _ = _fp8_cfg(1, 128, 8, 300, pad_frac=0.05)
     else:
         cfg = workloads.decode_bf16("cpu", batch=1, heads=128, pages_per_seq=8, topk=300, pad_frac=0.05)
-    if mode in ("eight_wavefronts", "wavefront_per_head_group"):
+    if mode != "first" and mode != "first_fp8":
         monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1" if mode == "eight_wavefronts" else "2")
     harness.lds_profile_start()
     try:

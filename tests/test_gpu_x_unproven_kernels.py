@@ -49,6 +49,17 @@ def test_logit_cap_many_heads_fp8(dev, splits):
     check_logit_cap(dev, 64, "fp8_e4m3_b128", 0.5, 0.2, 0.01, splits)
 
 
+@pytest.mark.parametrize("topk,n_splits,heads", [(1, 1, 40), (33, 1, 128), (64, 2, 65), (97, 1, 128), (129, 2, 128), (200, 3, 128),
+                                                 (1030, 1, 40), (2100, 2, 128), (2048, None, 128)])
+def test_head_group_kernel_fp8_pipeline(dev, monkeypatch, topk, n_splits, heads):
+    """The raw-record pipeline inside the wavefront-per-head-group kernel (FLAGTREE_SMLA_WIDE=2)."""
+    from flagtree_amd import workloads
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "2")
+    cfg = workloads.decode_fp8(dev, batch=3, heads=heads, pages_per_seq=40, topk=topk, pad_frac=0.0 if topk < 40 else 0.04)
+    out, lse = _fwd(cfg, n_splits=n_splits)
+    _check(cfg, out, lse)
+
+
 def test_fp8_many_heads_against_scalar_kernel_at_size(dev):
     """Batch 16 x 128 heads x 2048 records (64 tiles a list, two chunks): against the exact scalar
     kernel on two sequences and against the oracle on one."""
