@@ -51,6 +51,13 @@ def parse():
     return ap.parse_args()
 
 
+def many_heads_kernel(a, fmt):
+    """Name of the kernel a launch with more than 32 heads goes to under this run's switches."""
+    if a.wide == 2 or (a.wide == 1 and fmt == "bf16"):
+        return {1: "fwd_wide_kernel", 2: "fwd_group_kernel"}[a.wide]
+    return "fwd_tall_kernel"
+
+
 def measured_traffic(workload):
     """HBM bytes per launch of the workload's kernel as counted by rocprofv3 (FETCH_SIZE and
     WRITE_SIZE, each scaled by what the same counter reads for a plain copy of known size);
@@ -238,7 +245,7 @@ def main():
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = measured_traffic(a.workload)
     roof["traffic_source"] = TRAFFIC_NOTE
-    roof["kernel"] = ({1: "fwd_wide_kernel", 2: "fwd_group_kernel"}[a.wide] if a.wide and fmt == "bf16" else "fwd_tall_kernel") if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
+    roof["kernel"] = many_heads_kernel(a, fmt) if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
     roof["kernel_ms"] = kern_ms
     roof["other_bound"] = (dict(bound="hbm", achieved=nbytes / (kern_ms * 1e-3) / 1e9, peak=PEAK_HBM_GBS, unit="GB/s")
                            if not hbm_bound else
@@ -422,7 +429,7 @@ def bench_dense(a, torch, ft, workloads, dev):
                    "flops_per_step": flops, "bytes_per_step": nbytes},
         "roofline": {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": ach / PEAK_BF16_TFLOPS, "traffic": measured_traffic("decode_dense_bf16"),
-                     "traffic_source": TRAFFIC_NOTE, "kernel": "fwd_tall_kernel", "kernel_ms": kern_ms,
+                     "traffic_source": TRAFFIC_NOTE, "kernel": many_heads_kernel(a, "bf16"), "kernel_ms": kern_ms,
                      "other_bound": {"bound": "hbm", "achieved": nbytes / (kern_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                                      "unit": "GB/s", "frac": nbytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}},
         "timing": TIMING_NOTE}
