@@ -114,6 +114,25 @@ def test_workspace_and_split_planning(lib):
     assert lib.smla_plan_splits(2, 4, 16, 256) == 1            # fp32 plumbing path never splits
 
 
+def test_split_planning_follows_the_kernel_switches(lib, monkeypatch):
+    """A 128-heads-per-workgroup kernel has half as many (token, head block) units to fill the
+    device with, so the planner doubles the splits; the switches are read at every call.
+    (Without a GPU the library plans for 256 compute units.)"""
+    BF16, FP8 = 0, 1
+    monkeypatch.delenv("FLAGTREE_SMLA_WIDE", raising=False)
+    monkeypatch.delenv("FLAGTREE_SMLA_FEW_FP8", raising=False)
+    base = [lib.smla_plan_splits(BF16, 64, 128, 2048), lib.smla_plan_splits(FP8, 64, 128, 2048), lib.smla_plan_splits(FP8, 128, 16, 2048)]
+    assert base == [2, 2, 2]
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")                 # eight wavefronts: bf16 caches only
+    assert [lib.smla_plan_splits(BF16, 64, 128, 2048), lib.smla_plan_splits(FP8, 64, 128, 2048)] == [4, 2]
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "2")                 # a wavefront per head group: both formats
+    assert [lib.smla_plan_splits(BF16, 64, 128, 2048), lib.smla_plan_splits(FP8, 64, 128, 2048)] == [4, 4]
+    assert lib.smla_plan_splits(FP8, 128, 16, 2048) == 2           # few heads: not its business
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "0")
+    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")              # two workgroups per compute unit
+    assert lib.smla_plan_splits(FP8, 128, 16, 2048) == 4 and lib.smla_plan_splits(BF16, 64, 128, 2048) == 2
+
+
 def test_python_surface_rejects_bad_input():
     import flagtree_amd as ft
     q = torch.zeros((1, 2, 16, 576), dtype=torch.bfloat16)
