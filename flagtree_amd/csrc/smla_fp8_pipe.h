@@ -110,5 +110,16 @@ struct Convert {
   }
 };
 
+// Compile-time check of what Convert::store relies on: for every row0 = 8 * wave + l/32 the row xor
+// of row0 + 2k is that of row0 xor-ed with Layout::store_xor(k).
+template <typename Layout>
+constexpr bool layout_ok() {
+  for (int wave = 0; wave < 4; ++wave)
+    for (int g = 0; g < 2; ++g)
+      for (int k = 0; k < 4; ++k)
+        if (Layout::swz(8 * wave + g + 2 * k) != (Layout::swz(8 * wave + g) ^ Layout::store_xor(k))) return false;
+  return true;
+}
+
 }  // namespace fp8pipe
 }  // namespace smla

@@ -84,6 +84,7 @@ struct GroupLayout {
 using Fp8Pipe = fp8pipe::Pipe;
 using Fp8Convert = fp8pipe::Convert<GroupLayout>;
 static_assert(fp8pipe::kTN == kTN && fp8pipe::kMainStride == kMainStride && fp8pipe::kRopeBase == kRopeBase, "tile geometry");
+static_assert(fp8pipe::layout_ok<GroupLayout>(), "store_xor must describe this kernel's row xor");
 
 // A tile's rows go global -> LDS directly: one move brings the first 1 KB of a row (scalar row base
 // + per-lane chunk offset; lane l fetches chunk l ^ swz(row) so the row lands swizzled), one more

@@ -129,6 +129,7 @@ struct TallLayout {
 using Fp8Pipe = fp8pipe::Pipe;
 using Fp8Convert = fp8pipe::Convert<TallLayout>;
 static_assert(fp8pipe::kTN == kTN && fp8pipe::kMainStride == kMainStride && fp8pipe::kRopeBase == kRopeBase, "tile geometry");
+static_assert(fp8pipe::layout_ok<TallLayout>(), "store_xor must describe this kernel's row xor");
 
 // ---- per-tile math -------------------------------------------------------------------------
 // Softmax reference handling.  The fast pass takes each head's maximum over the first tile as
