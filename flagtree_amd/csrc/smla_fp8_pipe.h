@@ -75,18 +75,25 @@ struct Pipe {
 // use does not depend on row0: one per-lane offset then serves all four chunks.
 template <typename Layout>
 struct Convert {
-  uint4 v;
+  hw::u32x4 v;
   float sc;
   uint32_t o[8];
-  const uint8_t* raw;      // this wavefront's raw block
-  uint8_t* body;           // the tile body being written
+  uint32_t raw_lds;        // this wavefront's raw block
+  uint32_t body_lds;       // the tile body being written
   int wave, lane;
   __device__ __forceinline__ void load(int k) {
-    v = *reinterpret_cast<const uint4*>(raw + 16 * lane + 1024 * k);
-    sc = *reinterpret_cast<const float*>(raw + Pipe::kRawScales + 16 * (lane >> 5) + 4 * ((lane & 31) >> 3) + 32 * k);
+    v = hw::lds_read_u128(raw_lds + 16 * lane + 1024 * k);
+    sc = hw::lds_read_f32(raw_lds + Pipe::kRawScales + 16 * (lane >> 5) + 4 * ((lane & 31) >> 3) + 32 * k);
   }
+  // A lane turns 16 codes into the bf16 chunks 2*col and 2*col + 1 of its row, 16 bytes each, stored
+  // by two instructions.  A 16-byte store is served 16 lanes at a time, and sixteen EVEN chunks of a
+  // row cover only half the banks twice; so the lanes whose column has bit 3 set take their two
+  // chunks in the other order (`swap`): every instruction then writes sixteen chunks that differ
+  // modulo 16.  half(0) makes the chunk stored first, half(1) the other.
+  __device__ __forceinline__ bool swap() const { return (lane & 8) != 0; }
   __device__ __forceinline__ void half(int h) {
-    const uint32_t w[2] = {h == 0 ? v.x : v.z, h == 0 ? v.y : v.w};
+    const bool second = (h != 0) != swap();                        // which 8 codes: the first or the second half of the 16
+    const uint32_t w[2] = {second ? v[2] : v[0], second ? v[3] : v[1]};
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[k], false);
@@ -98,11 +105,11 @@ struct Convert {
   __device__ __forceinline__ void store(int k) {
     // tile row 8*wave + l/32 + 2k, chunks 2*col and 2*col + 1
     const int row0 = 8 * wave + (lane >> 5), col = lane & 31;
-    int off = row0 * kMainStride + (((2 * col) ^ Layout::swz(row0)) << 4);
+    int off = row0 * kMainStride + (((2 * col + (swap() ? 1 : 0)) ^ Layout::swz(row0)) << 4);
     hw::pin(off);                                                  // (worked out here, not kept in four registers from the top of the kernel)
     off = (off ^ (Layout::store_xor(k) << 4)) + 2 * k * kMainStride;
-    *reinterpret_cast<uint4*>(body + off) = make_uint4(o[0], o[1], o[2], o[3]);
-    *reinterpret_cast<uint4*>(body + (off ^ 16)) = make_uint4(o[4], o[5], o[6], o[7]);
+    hw::lds_write_b128(body_lds + off, hw::u32x4{o[0], o[1], o[2], o[3]});
+    hw::lds_write_b128(body_lds + (off ^ 16), hw::u32x4{o[4], o[5], o[6], o[7]});
   }
   __device__ __forceinline__ void whole_tile() {     // (one chunk at a time: where this is called, registers are scarce)
 #pragma unroll 1

@@ -26,6 +26,16 @@ __device__ __forceinline__ bf16x8 lds_read_b128(uint32_t a) {
 __device__ __forceinline__ void lds_write_b64(uint32_t a, u32x2 v) {
   *(__attribute__((address_space(3))) u32x2*)(a) = v;
 }
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+__device__ __forceinline__ void lds_write_b128(uint32_t a, u32x4 v) {
+  *(__attribute__((address_space(3))) u32x4*)(a) = v;
+}
+__device__ __forceinline__ u32x4 lds_read_u128(uint32_t a) {
+  return *(const __attribute__((address_space(3))) u32x4*)(a);
+}
+__device__ __forceinline__ float lds_read_f32(uint32_t a) {
+  return *(const __attribute__((address_space(3))) float*)(a);
+}
 // ds_read_b64_tr_b16: inside each group of 16 lanes, lane i receives element (i % 4) of the 8-byte
 // rows addressed by lanes (i / 4), (i / 4) + 4, (i / 4) + 8, (i / 4) + 12.
 __device__ __forceinline__ bf16x4 lds_read_tr16_b64(uint32_t a) {
@@ -116,7 +126,6 @@ __device__ __forceinline__ void store_b128_agent(float* p, f32x4 v) {
 // 16-byte loads at agent scope through a buffer descriptor: loads the compiler can see (it counts
 // them in flight and waits where a landing register is first read) that still carry sc1.
 typedef __amdgpu_buffer_rsrc_t buffer_rsrc;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 __device__ __forceinline__ buffer_rsrc make_rsrc(const void* wave_uniform_base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(wave_uniform_base), 0, 0x7fffffff, 0x00020000);
 }

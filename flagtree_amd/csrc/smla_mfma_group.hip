@@ -368,8 +368,8 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
                    ring + Fp8Pipe::kRawRing + (it & 1) * Fp8Pipe::kRawSlot + wave * Fp8Pipe::kRawWave, rope_addr(it), wave, ln);
       };
       [[maybe_unused]] auto convert_begin = [&](int it, int ln) {
-        cv.raw = &s_ring[Fp8Pipe::kRawRing + (it & 1) * Fp8Pipe::kRawSlot + wave * Fp8Pipe::kRawWave];
-        cv.body = &s_ring[(it % Fp8Pipe::kBodies) * kRopeBase];
+        cv.raw_lds = ring + Fp8Pipe::kRawRing + (it & 1) * Fp8Pipe::kRawSlot + wave * Fp8Pipe::kRawWave;
+        cv.body_lds = ring + (uint32_t)(it % Fp8Pipe::kBodies) * kRopeBase;
         cv.wave = wave; cv.lane = ln;
       };
       auto fetch_whole = [&](int it) {

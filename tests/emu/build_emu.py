@@ -26,9 +26,11 @@ def _stale(outputs, inputs):
 
 
 def build(verbose=False, force=False):
+    # every header a kernel source may include (the product's own smla_hw.h is shadowed by the emulator's)
     headers = [os.path.join(HERE, "emu_runtime.h"), os.path.join(HERE, "include", "smla_hw.h"),
-               os.path.join(HERE, "include", "hip", "hip_runtime.h"), os.path.join(CSRC, "smla_common.h"),
-               os.path.join(ROOT, "include", "flagtree_smla.h"), os.path.abspath(__file__)]
+               os.path.join(HERE, "include", "hip", "hip_runtime.h"), os.path.join(ROOT, "include", "flagtree_smla.h"),
+               os.path.abspath(__file__)]
+    headers += sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h") and f != "smla_hw.h")
     objs = []
     procs = []
     for src in SOURCES + ["emu_runtime.cc"]:

@@ -27,6 +27,25 @@ inline void lds_write_b64(uint32_t a, u32x2 v) {
   emu::lds_account(a, 8, 2);
   memcpy(emu::lds_ptr(a, 8), &v, 8);
 }
+inline void lds_write_b128(uint32_t a, u32x4 v) {
+  if (a & 15) emu::fail("ds_write_b128 at unaligned LDS address %u", a);
+  emu::lds_account(a, 16, 2);
+  memcpy(emu::lds_ptr(a, 16), &v, 16);
+}
+inline u32x4 lds_read_u128(uint32_t a) {
+  if (a & 15) emu::fail("ds_read_b128 at unaligned LDS address %u", a);
+  emu::lds_account(a, 16, 0);
+  u32x4 v;
+  memcpy(&v, emu::lds_ptr(a, 16), 16);
+  return v;
+}
+inline float lds_read_f32(uint32_t a) {
+  if (a & 3) emu::fail("ds_read_b32 at unaligned LDS address %u", a);
+  emu::lds_account(a, 4, 0);
+  float v;
+  memcpy(&v, emu::lds_ptr(a, 4), 4);
+  return v;
+}
 // ds_read_b64_tr_b16: inside each group of 16 lanes, lane i receives element (i % 4) of the 8-byte
 // rows addressed by lanes (i / 4), (i / 4) + 4, (i / 4) + 8, (i / 4) + 12 of the group.
 inline bf16x4 lds_read_tr16_b64(uint32_t a) {
