@@ -599,7 +599,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   }
   hw::wave_lds_order();
   const int n_rows = max(0, min(32, p.n_heads - head0));           // head rows that exist (wave-uniform)
-  constexpr int kStageStride = kDv + 8;                            // floats per staged row (+32 B pad)
+  constexpr int kStageStride = kDv + 4;                            // floats per staged row (+16 B pad: the four row groups a store touches start 16 banks apart)
   static_assert(4 * 16 * kStageStride * 4 <= kSlots * kTileBytes, "the staged blocks must fit the ring area");
   float* stage = reinterpret_cast<float*>(&s_ring[0]) + wave * 16 * kStageStride;
   const int col8 = 8 * lane_e;                                     // this lane's 8 output columns when rows are read back
