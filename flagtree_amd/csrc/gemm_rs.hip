@@ -352,14 +352,16 @@ __device__ __forceinline__ void gemm_big_tile(const uint16_t* __restrict__ x, co
     for (int r = 0; r < 16; ++r) {
       const int row = 8 * (r >> 2) + 4 * g + (r & 3);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) stage[row * kStage2Floats + 32 * j + c32] = acc[i][j][r];
+      // (a row is exactly the 64 banks wide, and a store's two half-wavefronts write rows 4 apart:
+      // rows with bit 2 set keep their two 32-float halves swapped, so the halves land on different banks)
+      for (int j = 0; j < 2; ++j) stage[row * kStage2Floats + ((32 * j + c32) ^ (32 * g))] = acc[i][j][r];
     }
     __builtin_amdgcn_wave_barrier();                    // (the area is the wavefront's own; its LDS operations complete in order)
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
       const int row = 4 * p + rsub;
       const int m = m0 + 32 * MI * wm + 32 * i + row;
-      const float4 v = *reinterpret_cast<const float4*>(stage + row * kStage2Floats + col4);
+      const float4 v = *reinterpret_cast<const float4*>(stage + row * kStage2Floats + (col4 ^ (32 * ((row >> 2) & 1))));
       const g_f32x4 zz = z[p];
       const int chunk = m / rows_per_chunk;
       uint16_t* o = out + (size_t)chunk * chunk_stride + (size_t)(m - chunk * rows_per_chunk) * N + n;
