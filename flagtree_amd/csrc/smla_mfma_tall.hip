@@ -680,7 +680,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   const float l_tot = s_x[wave][c32_e] + s_x[partner][c32_e];
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const float lse_nat = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
-  constexpr int kStageStride = kDvHalf + 4;                        // floats per staged row (+16 B pad)
+  constexpr int kStageStride = kDvHalf + 8;                        // floats per staged row (+32 B pad: a store's two half-wavefronts write rows 4 apart, which then land 32 banks apart)
   static_assert(4 * 32 * kStageStride * 4 <= kRingBytes, "the staged blocks must fit the ring area");
   float* stage = reinterpret_cast<float*>(&s_ring[0]) + wave * 32 * kStageStride;
 #pragma unroll

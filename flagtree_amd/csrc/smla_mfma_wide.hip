@@ -52,7 +52,7 @@ enum { kPassFast = 0, kPassMax = 1, kPassFinal = 2 };
 constexpr int kRingBytes = kSlots * kTileBytes;                 // 129 024
 constexpr int kPOff = kRingBytes;                               // P buffers [tile parity][head group]
 constexpr int kLdsBytes = kPOff + 2 * 4 * kPBytes;              // 141 312
-constexpr int kStageStride = kDvHalf + 4;                       // floats per staged output row (+16 B pad)
+constexpr int kStageStride = kDvHalf + 8;                       // floats per staged output row (+32 B pad: rows 4 apart land 32 banks apart)
 static_assert(8 * 16 * kStageStride * 4 <= kLdsBytes, "the epilogue stages 16 rows x 256 columns per wavefront");
 static_assert(kBtLdsMax * 4 <= kTileBytes, "the page-table row is staged in one ring slot");
 
