@@ -63,9 +63,11 @@ __device__ __forceinline__ void wave_lds_order() {}
 // (wave-uniform, goes through M0).  They complete in issue order and are counted by vmcnt like
 // any other vector memory operation; nothing orders them against LDS reads but wait_vmcnt and
 // a barrier.  Issued from inline assembly (no register output) so that the compiler does not
-// serialise them against LDS reads of other ring slots.
+// serialise them against LDS reads of other ring slots.  The s_nop is the wait state the ISA asks
+// for between a scalar write of M0 and a memory instruction that uses it as its LDS base (the
+// compiler inserts it in its own code; inside an asm statement nobody does).
 __device__ __forceinline__ void dma_b128(const void* lane_src, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(lane_src), "s"(lds_base) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(lane_src), "s"(lds_base) : "memory", "m0");
 }
 // A move in which only lanes 0 .. N-1 take part (the others' LDS pieces stay as they are).  The
 // execution mask is narrowed and restored around the instruction right here, so that no branch
@@ -75,15 +77,15 @@ template <int N>
 __device__ __forceinline__ void dma_b128_first_lanes(const void* lane_src, uint32_t lds_base) {
   static_assert(N > 0 && N < 32, "the mask is written as a 32-bit literal");
   uint64_t saved;
-  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %3\n\ts_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b64 exec, %0"
+  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %3\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b64 exec, %0"
                : "=&s"(saved) : "v"(lane_src), "s"(lds_base), "n"((1u << N) - 1u) : "memory", "m0");
 }
 // scalar base + per-lane byte offset
 __device__ __forceinline__ void dma_b128(uint32_t lane_off, uint64_t wave_base, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(wave_base), "s"(lds_base) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(wave_base), "s"(lds_base) : "memory", "m0");
 }
 __device__ __forceinline__ void dma_b32(const void* lane_src, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(lane_src), "s"(lds_base) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(lane_src), "s"(lds_base) : "memory", "m0");
 }
 
 // s_waitcnt vmcnt(N): at most N of this wavefront's vector memory operations still in flight

@@ -133,6 +133,18 @@ def test_one_wavefront_per_simd_kernels_use_the_whole_register_file():
     assert len(big) == 1 and big[0]["VGPRs"] + big[0]["AGPRs"] <= 128 and big[0]["LDS Size"] == 128 * 1024, big
 
 
+@pytest.mark.parametrize("source", [s for s in build.SOURCES if s != "smla_api.hip"])
+def test_every_global_to_lds_move_has_its_m0_wait_state(source):
+    """The ISA asks for one wait state between a scalar write of M0 and a memory instruction that
+    takes its LDS base from M0.  The moves are issued from inline assembly, where the compiler's
+    hazard pass does not look, so the s_nop is written out; this checks the compiled code."""
+    _, asm = _compile(source)
+    lines = [l.strip() for l in asm.splitlines()]
+    moves = [i for i, l in enumerate(lines) if l.startswith("global_load_lds")]
+    for i in moves:
+        assert lines[i - 1].startswith("s_nop") and lines[i - 2].startswith("s_mov_b32 m0"), (source, lines[i - 3:i + 1])
+
+
 _LOAD_MNEMONIC = re.compile(r"\b(global_load|buffer_load|flat_load|scratch_load|ds_read|ds_load|s_load|s_buffer_load)")
 
 
