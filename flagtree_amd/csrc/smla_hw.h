@@ -120,9 +120,12 @@ __device__ __forceinline__ void shift_in_eq_u32(uint32_t& mask, uint32_t x, uint
   asm("v_cmp_eq_u32 vcc, %1, %2\n\ts_nop 1\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc" : "+v"(mask) : "v"(x), "v"(y) : "vcc");
 }
 
-// 16-byte store at agent scope (sc1: written through to the L2 every CU of the XCD shares)
+// 16-byte store at agent scope (sc1: written through to the L2 every CU of the XCD shares).
+// The s_nop covers the two wait states the ISA asks for between a store of more than 8 bytes and
+// a vector instruction that overwrites the registers holding its data (the compiler, which would
+// insert them for a store of its own, is free to reuse those registers right after the statement).
 __device__ __forceinline__ void store_b128_agent(float* p, f32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }
 
 // 16-byte loads at agent scope through a buffer descriptor: loads the compiler can see (it counts

@@ -145,6 +145,17 @@ def test_every_global_to_lds_move_has_its_m0_wait_state(source):
         assert lines[i - 1].startswith("s_nop") and lines[i - 2].startswith("s_mov_b32 m0"), (source, lines[i - 3:i + 1])
 
 
+@pytest.mark.parametrize("source", [s for s in build.SOURCES if s != "smla_api.hip"])
+def test_agent_scope_stores_from_assembly_keep_their_data_registers(source):
+    """A store of more than 8 bytes reads its data registers for two more wait states; the 16-byte
+    agent-scope stores are issued from inline assembly, so the s_nop is written out."""
+    _, asm = _compile(source)
+    lines = [l.strip() for l in asm.splitlines()]
+    for i, l in enumerate(lines):
+        if l.startswith("global_store_dwordx4") and " sc1" in l and lines[i - 1].startswith(";;#ASMSTART"):
+            assert lines[i + 1].startswith("s_nop 1"), (source, lines[i - 1:i + 3])
+
+
 _LOAD_MNEMONIC = re.compile(r"\b(global_load|buffer_load|flat_load|scratch_load|ds_read|ds_load|s_load|s_buffer_load)")
 
 
