@@ -243,7 +243,8 @@ def main():
     else:
         roof = dict(bound="mfma", achieved=flops / (kern_ms * 1e-3) / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = measured_traffic(a.workload)
+    # (the stored counter figures were taken on the default kernels: none for a kernel behind a switch)
+    roof["traffic"] = None if (a.wide or a.few_fp8) else measured_traffic(a.workload)
     roof["traffic_source"] = TRAFFIC_NOTE
     roof["kernel"] = many_heads_kernel(a, fmt) if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
     roof["kernel_ms"] = kern_ms
@@ -428,7 +429,7 @@ def bench_dense(a, torch, ft, workloads, dev):
         "config": {"workload": "decode_dense_bf16", "batch": B, "heads": H, "context": ctx, "page_size": cfg["page_size"],
                    "flops_per_step": flops, "bytes_per_step": nbytes},
         "roofline": {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": ach / PEAK_BF16_TFLOPS, "traffic": measured_traffic("decode_dense_bf16"),
+                     "frac": ach / PEAK_BF16_TFLOPS, "traffic": None if a.wide else measured_traffic("decode_dense_bf16"),
                      "traffic_source": TRAFFIC_NOTE, "kernel": many_heads_kernel(a, "bf16"), "kernel_ms": kern_ms,
                      "other_bound": {"bound": "hbm", "achieved": nbytes / (kern_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                                      "unit": "GB/s", "frac": nbytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}},
