@@ -69,7 +69,17 @@ struct Wave {
   unsigned long long gen = 0;      // completed rendezvous
   uint32_t tag = 0;
   bool lane_live[kWave];
+  // the lanes that took part in the last rendezvous of each parity: what a lane reads after a
+  // rendezvous must not depend on which of the others have meanwhile run on and left the kernel
+  unsigned long long took_part[2] = {0, 0};
   alignas(64) uint8_t slot[2][kWave][kSlotBytes];
+  void complete() {
+    unsigned long long m = 0;
+    for (int l = 0; l < kWave; ++l) m |= (unsigned long long)lane_live[l] << l;
+    took_part[gen & 1] = m;
+    arrived = 0;
+    gen++;
+  }
 };
 
 namespace {
@@ -100,7 +110,7 @@ void leave_wave(Fiber* f) {
   w->lane_live[f->lane.lane] = false;
   w->live--;
   // a rendezvous the others are waiting in may now be complete
-  if (w->live > 0 && w->arrived == w->live) { w->arrived = 0; w->gen++; }
+  if (w->live > 0 && w->arrived == w->live) w->complete();
   g_block.live--;
   if (g_block.live > 0 && g_block.arrived == g_block.live) { g_block.arrived = 0; g_block.gen++; }
 }
@@ -156,8 +166,10 @@ void run_block(Dim3 bidx) {
     f.stack = get_stack(i);
     prepare(&f);
   }
-  for (Wave& w : g_block.waves)
+  for (Wave& w : g_block.waves) {
     for (int l = w.n_lanes; l < kWave; ++l) w.lane_live[l] = false;
+    w.took_part[0] = w.took_part[1] = w.n_lanes == kWave ? ~0ull : (1ull << w.n_lanes) - 1ull;
+  }
   // round-robin until every lane has left; a full round without any lane finishing or any
   // rendezvous completing means the lanes are waiting for each other in different places
   unsigned long long idle_rounds = 0;
@@ -216,9 +228,9 @@ int wave_rendezvous(const void* post, size_t bytes, uint32_t tag) {
          "a collective inside divergent control flow", g_block_idx.x, g_block_idx.y, g_block_idx.z,
          f->lane.flat / kWave, w->tag, tag);
   w->arrived++;
+  f->lane.parity = parity;
   if (w->arrived == w->live) {
-    w->arrived = 0;
-    w->gen++;
+    w->complete();
   } else {
     f->wait_gen = &w->gen;
     f->wait_val = my_gen;
@@ -228,7 +240,7 @@ int wave_rendezvous(const void* post, size_t bytes, uint32_t tag) {
 }
 
 const uint8_t* wave_slot(int parity, int lane) { return g_cur->lane.wave->slot[parity][lane]; }
-bool wave_lane_live(int lane) { return g_cur->lane.wave->lane_live[lane]; }
+bool wave_lane_live(int lane) { return (g_cur->lane.wave->took_part[g_cur->lane.parity] >> lane) & 1; }
 
 void block_barrier() {
   g_work.barriers_lane_calls++;

@@ -32,6 +32,7 @@ struct Lane {
   int lane;                            // lane id in its wavefront
   int flat;                            // thread id in the workgroup
   Wave* wave;
+  int parity = 0;                      // slot set of the last rendezvous this lane went through
 };
 
 Lane* self();                          // the lane that is running now
@@ -44,7 +45,7 @@ Dim3 grid_dim();
 // Returns the parity of the slot set posted for this rendezvous.
 int wave_rendezvous(const void* post, size_t bytes, uint32_t tag);
 const uint8_t* wave_slot(int parity, int lane);      // what `lane` posted (valid until the next rendezvous but one)
-bool wave_lane_live(int lane);                       // lane exists and has not left the kernel
+bool wave_lane_live(int lane);                       // `lane` took part in the calling lane's last rendezvous
 void block_barrier();
 
 // LDS arena: every __shared__ object lives in the ELF section "emu_lds"

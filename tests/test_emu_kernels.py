@@ -587,6 +587,22 @@ def test_topk_indices_exact(rows, n, k):
     assert np.array_equal(to_np(out), oracle.topk_indices(to_np(scores), k, to_np(lens)))
 
 
+@pytest.mark.parametrize("n,length,k", [(65537, 300, 64), (65537, 10117, 300), (70001, 70001, 2048), (65536, 1000, 64)])
+def test_topk_indices_with_tied_values_in_long_rows(n, length, k):
+    """Scores rounded to quarters, so that the k-th place is shared by many entries, in rows above
+    and at the length where the launcher changes kernels.  In the kernel for long rows the vote
+    that ranks the tied entries is the last thing a lane does: lanes that leave the kernel right
+    after it must still count in the vote as the lanes behind them read it (the emulator once
+    dropped them)."""
+    g = torch.Generator().manual_seed(n + length + k)
+    scores = (torch.randn((2, n), generator=g) * 4).round() / 4
+    lens = torch.tensor([length, max(1, length // 3)], dtype=torch.int32)
+    out = torch.full((2, k), -9, dtype=torch.int32)
+    rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), 2, n, n, k, None)
+    assert rc == 0
+    assert np.array_equal(to_np(out), oracle.topk_indices(to_np(scores), k, to_np(lens)))
+
+
 @pytest.mark.parametrize("m,n,k,chunks", [(256, 256, 128, 2), (128, 512, 192, 1), (384, 256, 64, 3), (512, 256, 128, 4),
                                           (2048, 256, 64, 8),      # 8 tiles on 16 units: every tile as two half tiles
                                           (2048, 768, 128, 2)])    # 24 tiles: 16 whole + 8 split into 16 half tiles

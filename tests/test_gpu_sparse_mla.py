@@ -273,7 +273,8 @@ def test_topk_indices_exact(dev, n, k, quant):
 @pytest.mark.parametrize("rows,n,k,quant", [(1100, 4096, 300, 0),      # many short rows
                                              (1030, 5000, 512, 4),      # many rows, four rounds a wavefront, the last ones partial
                                              (1024, 6000, 5500, 0),     # list too long for the LDS staging
-                                             (3, 16384, 9000, 16), (2, 40000, 30000, 0), (2, 70000, 100, 2)])
+                                             (3, 16384, 9000, 16), (2, 40000, 30000, 0), (2, 70000, 100, 2),
+                                             (6, 65537, 64, 4)])        # the first length of the kernel for long rows, tied values
 def test_topk_indices_shapes(dev, rows, n, k, quant):
     """Every kernel variant the launcher picks (by row count and length), with context lengths that
     leave wavefronts without entries, rounds partly filled and rows empty."""
