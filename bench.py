@@ -48,6 +48,9 @@ def parse():
                          "2: a wavefront per 32 heads; opt-in until measured)")
     ap.add_argument("--few-fp8", action="store_true",
                     help="decode_fp8 on the two-workgroups-per-CU kernel (sets FLAGTREE_SMLA_FEW_FP8=1; opt-in until measured)")
+    ap.add_argument("--token-bands", action="store_true",
+                    help="each XCD takes a contiguous band of tokens instead of every eighth one (sets "
+                         "FLAGTREE_SMLA_TOKEN_BANDS=1; for prefill_causal_bf16; opt-in until measured)")
     return ap.parse_args()
 
 
@@ -125,6 +128,8 @@ def main():
         os.environ["FLAGTREE_SMLA_FEW_FP8"] = "1"
     if a.wide:
         os.environ["FLAGTREE_SMLA_WIDE"] = str(a.wide)
+    if a.token_bands:
+        os.environ["FLAGTREE_SMLA_TOKEN_BANDS"] = "1"
     import torch
     import flagtree_amd as ft
     from flagtree_amd import workloads
@@ -244,7 +249,7 @@ def main():
         roof = dict(bound="mfma", achieved=flops / (kern_ms * 1e-3) / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
     # (the stored counter figures were taken on the default kernels: none for a kernel behind a switch)
-    roof["traffic"] = None if (a.wide or a.few_fp8) else measured_traffic(a.workload)
+    roof["traffic"] = None if (a.wide or a.few_fp8 or a.token_bands) else measured_traffic(a.workload)
     roof["traffic_source"] = TRAFFIC_NOTE
     roof["kernel"] = many_heads_kernel(a, fmt) if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
     roof["kernel_ms"] = kern_ms
@@ -266,7 +271,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": a.workload, "batch": cfg["q"].shape[0], "heads": H, "topk": K,
                    "n_valid": n_valid, "kv_format": fmt, "page_size": cfg["page_size"],
-                   "n_splits": n_splits, "input_sets": len(sets),
+                   "n_splits": n_splits, "input_sets": len(sets), "token_bands": bool(a.token_bands),
                    "flops_per_step": flops, "bytes_per_step": nbytes},
         "hbm_gbs": gbs, "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
         "pct_hbm_peak": 100.0 * gbs / PEAK_HBM_GBS,

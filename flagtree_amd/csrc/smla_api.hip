@@ -41,6 +41,13 @@ bool few_fp8_enabled() {
   return e != nullptr && e[0] == '1';
 }
 
+// FLAGTREE_SMLA_TOKEN_BANDS=1 gives each XCD a contiguous band of tokens instead of every eighth
+// token (for causal prefill; see token_of).
+bool token_bands_enabled() {
+  const char* e = getenv("FLAGTREE_SMLA_TOKEN_BANDS");
+  return e != nullptr && e[0] == '1';
+}
+
 int device_cus() {
   static int cus = 0;
   if (cus == 0) {
@@ -148,6 +155,7 @@ static int fill_params(Params& p, const void* q, const void* kv, const int32_t* 
   p.page_size = block_table ? page_size : 1; p.bt_stride = block_table ? bt_stride : 0;
   p.n_splits = 1; p.split_len = topk;
   p.kv_seq_stride = kv_seq_stride; p.kv_rows = kv_rows; p.sm_scale = sm_scale; p.logit_cap = 0.f;
+  p.token_band = token_bands_enabled() ? (n_tokens + 7) / 8 : 0;
   return SMLA_OK;
 }
 

@@ -34,7 +34,17 @@ struct Params {
   int64_t kv_seq_stride, kv_rows;
   float sm_scale;
   float logit_cap;              // > 0: every scaled score s becomes logit_cap * tanh(s / logit_cap) before the softmax
+  int32_t token_band;           // 0: tokens dealt to the 8 XCDs in turn; > 0: XCD x takes tokens x*token_band .. (x+1)*token_band - 1
 };
+
+// Which token a workgroup works on.  Block ids are dealt round-robin to the 8 XCDs (`xcd` = id % 8,
+// `round` = how many tokens that XCD has been given before).  Dealing tokens in turn keeps the
+// XCDs level whatever the lists hold.  Contiguous bands (opt-in) are for causal prefill, where
+// token t selects among rows 0 .. t: an XCD then gathers from the rows before its band's end
+// instead of from the whole cache, so that the early bands' rows stay in its own L2.
+__device__ __forceinline__ int token_of(const Params& p, int xcd, int round) {
+  return p.token_band > 0 ? xcd * p.token_band + round : round * 8 + xcd;     // (round < token_band by the grid's size)
+}
 
 // The capped score in the base-2 units the softmax works in:
 //   log2(e) * cap * tanh(x / cap),  x = raw dot product * sm_scale,

@@ -235,7 +235,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int hb = slot % n_hblocks;
   const int sp = (slot / n_hblocks) % p.n_splits;
-  const int t = (slot / (n_hblocks * p.n_splits)) * 8 + xcd;
+  const int t = token_of(p, xcd, slot / (n_hblocks * p.n_splits));
   if (t >= p.n_tokens) return;
   const int seq = t / p.tokens_per_seq;
   const int head0 = hb * 128 + wave * 32;                         // first head of this wavefront

@@ -322,6 +322,26 @@ def test_causal_prefill_reduced():
     _check(cfg, out, lse)
 
 
+@pytest.mark.parametrize("wide", ["0", "1", "2"])
+@pytest.mark.parametrize("heads,n_splits", [(128, 1), (128, 2), (16, 1), (16, 3)])
+def test_token_bands_only_change_which_workgroup_takes_a_token(heads, n_splits, wide, monkeypatch):
+    """FLAGTREE_SMLA_TOKEN_BANDS=1 hands each XCD a contiguous band of tokens instead of every
+    eighth one: every token is still computed once, by the same code, so the results are the same
+    bits (43 tokens: bands of 6, the last one short, some workgroups without a token)."""
+    from flagtree_amd import workloads
+    if heads == 16 and wide != "0":
+        pytest.skip("the 128-heads kernels do not take 16 heads")
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", wide)
+    cfg = workloads.prefill_causal_bf16("cpu", tokens=43, heads=heads, topk=300 if n_splits > 1 else 48)
+    out0, lse0, rc = harness.forward(cfg, n_splits=n_splits)
+    assert rc == 0
+    monkeypatch.setenv("FLAGTREE_SMLA_TOKEN_BANDS", "1")
+    out1, lse1, rc = harness.forward(cfg, n_splits=n_splits)
+    assert rc == 0
+    assert torch.equal(out0.view(torch.int16), out1.view(torch.int16)) and torch.equal(lse0, lse1)
+    _check(cfg, out1, lse1)
+
+
 @pytest.mark.parametrize("heads", [128, 16])
 def test_edge_cases(heads):
     g = torch.Generator().manual_seed(7)

@@ -1,6 +1,7 @@
 """GPU parity of the kernel paths that have not been timed or run on hardware yet: the many-heads
 kernel over an fp8 cache (raw records by global -> LDS moves, converted LDS -> LDS) and the two
-opt-in second designs (FLAGTREE_SMLA_FEW_FP8, FLAGTREE_SMLA_WIDE).  The file sorts after the other
+opt-in second designs (FLAGTREE_SMLA_FEW_FP8, FLAGTREE_SMLA_WIDE) and the opt-in token order
+(FLAGTREE_SMLA_TOKEN_BANDS).  The file sorts after the other
 GPU test files on purpose: under `pytest -x` a failure here cannot hide the results of the paths
 the defaults rest on.  Same bars: out max-abs <= 1e-2, lse <= 1e-3 against the float64 oracle."""
 import numpy as np
@@ -198,3 +199,18 @@ def test_128_heads_kernel_prefill_and_redo(dev, wide_kernel):
         out, lse = _fwd(cfg, n_splits=ns)
         assert max_abs(to_np(lse).reshape(rl.shape), rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
         assert max_abs(to_np(out).reshape(ro.shape), ro) <= 1.2e-2 * max(1.0, float(np.abs(ro).max()))
+
+
+# ---- contiguous token bands per XCD (opt-in) ---------------------------------------------------
+
+@pytest.mark.parametrize("heads,n_splits,tokens", [(128, 1, 320), (128, 2, 43), (16, 1, 171), (16, 3, 43)])
+def test_token_bands_give_the_same_bits(dev, monkeypatch, heads, n_splits, tokens):
+    """FLAGTREE_SMLA_TOKEN_BANDS=1 only changes which workgroup takes which token (an XCD gets a
+    contiguous band instead of every eighth token): out and lse must not change by a bit."""
+    from flagtree_amd import workloads
+    cfg = workloads.prefill_causal_bf16(dev, tokens=tokens, heads=heads, topk=300 if n_splits > 1 else 128)
+    out0, lse0 = _fwd(cfg, n_splits=n_splits)
+    monkeypatch.setenv("FLAGTREE_SMLA_TOKEN_BANDS", "1")
+    out1, lse1 = _fwd(cfg, n_splits=n_splits)
+    assert torch.equal(out0.view(torch.int16), out1.view(torch.int16)) and torch.equal(lse0, lse1)
+    _check(cfg, out1, lse1)
