@@ -12,10 +12,11 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 CSRC = os.path.join(ROOT, "flagtree_amd", "csrc")
 LIB_PATH = os.path.join(HERE, "libflagtree_smla_emu.so")
 SOURCES = ["smla_api.hip", "smla_scalar.hip", "smla_mfma_tall.hip", "smla_mfma_short.hip", "smla_mfma_few_fp8.hip", "smla_mfma_wide.hip", "smla_mfma_group.hip", "gemm_rs.hip", "topk_select.hip"]
+HW_MODEL = os.path.join(os.path.dirname(HERE), "hw_model")      # probes of single instructions, built for both sides
 CXX = os.environ.get("EMU_CXX", "/opt/rocm/llvm/bin/clang++")
 FLAGS = ["-x", "c++", "-std=c++17", "-O2", "-g1", "-fPIC", "-ffp-contract=off", "-fno-strict-aliasing",
          "-Wno-unused-value", "-Wno-pass-failed", "-Wno-unknown-attributes", "-Wno-ignored-attributes",
-         "-I", os.path.join(HERE, "include"), "-I", CSRC]
+         "-I", os.path.join(HERE, "include"), "-I", CSRC, "-I", HW_MODEL]
 
 
 def _stale(outputs, inputs):
@@ -33,8 +34,9 @@ def build(verbose=False, force=False):
     headers += sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h") and f != "smla_hw.h")
     objs = []
     procs = []
-    for src in SOURCES + ["emu_runtime.cc"]:
-        path = os.path.join(HERE if src.endswith(".cc") else CSRC, src)
+    headers.append(os.path.join(HW_MODEL, "primitives.h"))
+    for src in SOURCES + ["primitives.hip", "emu_runtime.cc"]:
+        path = os.path.join(HERE if src.endswith(".cc") else (HW_MODEL if src == "primitives.hip" else CSRC), src)
         obj = os.path.join(HERE, "build", src + ".o")
         objs.append(obj)
         if not force and not _stale([obj], [path] + headers):
