@@ -645,7 +645,8 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   // ---- split merge inside the launch (protocol and failure handling: ws_arrive / ws_wait_published
   // in smla_common.h; described in smla_mfma_tall.hip)
   unsigned long long* word = p.counters + (size_t)t * n_hblocks + hb;
-  const int role = s_nvalid;                                       // ticket taken at the top of the epilogue
+  __syncthreads();                                                 // the ticket lane 0 of wavefront 0 took at the top of the epilogue is in s_nvalid
+  const int role = s_nvalid;
   auto give_up = [&]() {
 #pragma unroll
     for (int ht = 0; ht < 2; ++ht)

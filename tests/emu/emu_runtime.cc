@@ -99,6 +99,7 @@ Dim3 g_block_idx, g_block_dim, g_grid_dim;
 const std::function<void()>* g_body = nullptr;
 int g_dma_eager = 0;
 unsigned g_order_seed = 0;
+unsigned g_wave_skew = 0;
 unsigned long long g_launches = 0;
 int g_cu_count = 256;
 std::vector<char*> g_stacks;
@@ -143,6 +144,45 @@ void prepare(Fiber* f) {
   f->sp = s;
 }
 
+// One round over the lanes of wavefront `wv` only; true when any of them ran.
+bool run_wave_once(size_t wv) {
+  bool ran = false;
+  const size_t f0 = wv * kWave, f1 = std::min(g_block.fibers.size(), f0 + kWave);
+  for (size_t i = f0; i < f1; ++i) {
+    Fiber& f = g_block.fibers[i];
+    if (f.done) continue;
+    if (f.wait_gen != nullptr && *f.wait_gen == f.wait_val) continue;
+    f.wait_gen = nullptr;
+    g_cur = &f;
+    emu_switch(&g_sched_sp, f.sp);
+    ran = true;
+  }
+  return ran;
+}
+
+// Skewed schedule: the wavefronts of a workgroup do not advance together.  A wavefront drawn at
+// random runs alone for a random stretch, up to the point where it can only wait for the others
+// (a workgroup barrier, the end of the kernel), then another is drawn.  On the hardware nothing
+// but barriers keeps wavefronts in step; a kernel that relies on them advancing together (a ring
+// slot refilled while a slower wavefront still reads it, a flag read before it is written)
+// passes under the even schedule and fails under this one.
+void run_block_skewed(Dim3 bidx) {
+  std::mt19937 rng(g_wave_skew * 2654435761u + bidx.x * 40503u + bidx.y * 97u + bidx.z);
+  const size_t n_waves = g_block.waves.size();
+  unsigned long long stuck_draws = 0;
+  while (g_block.live > 0) {
+    const size_t wv = rng() % n_waves;
+    const unsigned stretch = 1u + rng() % ((rng() & 3) == 0 ? 4096u : 48u);      // mostly short, now and then as far as it gets
+    bool any = false;
+    for (unsigned r = 0; r < stretch && run_wave_once(wv); ++r) any = true;
+    if (any) {
+      stuck_draws = 0;
+    } else if (++stuck_draws > 64 * n_waves) {                                   // every wavefront drawn many times, none could run
+      fail("deadlock in block (%u,%u,%u): %d lanes wait at barriers that cannot complete", bidx.x, bidx.y, bidx.z, g_block.live);
+    }
+  }
+}
+
 void run_block(Dim3 bidx) {
   const unsigned n = g_block_dim.x * g_block_dim.y * g_block_dim.z;
   const unsigned n_waves = (n + kWave - 1) / kWave;
@@ -169,6 +209,11 @@ void run_block(Dim3 bidx) {
   for (Wave& w : g_block.waves) {
     for (int l = w.n_lanes; l < kWave; ++l) w.lane_live[l] = false;
     w.took_part[0] = w.took_part[1] = w.n_lanes == kWave ? ~0ull : (1ull << w.n_lanes) - 1ull;
+  }
+  if (g_wave_skew != 0 && n_waves > 1) {
+    run_block_skewed(bidx);
+    g_cur = nullptr;
+    return;
   }
   // round-robin until every lane has left; a full round without any lane finishing or any
   // rendezvous completing means the lanes are waiting for each other in different places
@@ -406,6 +451,7 @@ void launch(Dim3 grid, Dim3 block, const std::function<void()>& body) {
 extern "C" {
 void emu_set_dma_mode(int eager) { emu::g_dma_eager = eager; }
 void emu_set_block_order(unsigned seed) { emu::g_order_seed = seed; }
+void emu_set_wave_skew(unsigned seed) { emu::g_wave_skew = seed; }
 unsigned long long emu_launch_count(void) { return emu::g_launches; }
 void emu_set_cu_count(int n) { emu::g_cu_count = n; }
 void emu_set_lds_profile(int on) {

@@ -163,7 +163,7 @@ if __name__ == "__main__":
     for name in names:
         for end in (True, False):
             print(f"guarded case {name} ({'end' if end else 'start'} of every buffer at a page edge)", flush=True)
-            for eager in (False, True):
-                harness.configure(dma_eager=eager)
+            for eager, skew in ((False, 0), (True, 11)):      # (the second pass also with the wavefronts of a workgroup out of step)
+                harness.configure(dma_eager=eager, wave_skew_seed=skew)
                 CASES[name](end)
     print("ok")

@@ -31,6 +31,7 @@ def lib():
             fn.argtypes = args
         l.emu_set_dma_mode.argtypes = [ctypes.c_int]
         l.emu_set_block_order.argtypes = [ctypes.c_uint]
+        l.emu_set_wave_skew.argtypes = [ctypes.c_uint]
         l.emu_launch_count.restype = ctypes.c_ulonglong
         l.emu_set_cu_count.argtypes = [ctypes.c_int]
         l.emu_set_lds_profile.argtypes = [ctypes.c_int]
@@ -41,10 +42,11 @@ def lib():
     return _lib
 
 
-def configure(dma_eager=False, block_order_seed=0):
+def configure(dma_eager=False, block_order_seed=0, wave_skew_seed=0):
     l = lib()
     l.emu_set_dma_mode(1 if dma_eager else 0)
     l.emu_set_block_order(block_order_seed)
+    l.emu_set_wave_skew(wave_skew_seed)
 
 
 def lds_profile_start():

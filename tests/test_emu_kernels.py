@@ -37,6 +37,16 @@ def _emulator():
     harness.configure()
 
 
+@pytest.fixture(params=[0, 3], ids=["wavefronts_in_step", "wavefronts_skewed"])
+def schedule(request):
+    """For tests that make a single call: once with a workgroup's wavefronts advancing together,
+    once with them running one at a time for random stretches (only barriers keep them in step on
+    the hardware)."""
+    harness.configure(wave_skew_seed=request.param)
+    yield
+    harness.configure()
+
+
 def _check(cfg, out, lse, out_tol=OUT_TOL, lse_tol=LSE_TOL):
     ro, rl = run_oracle(cfg)
     H = cfg["q"].shape[-2]
@@ -47,11 +57,13 @@ def _check(cfg, out, lse, out_tol=OUT_TOL, lse_tol=LSE_TOL):
 
 
 def _forward_all_ways(cfg, n_splits, **kw):
-    """Forward under every emulator setting; results must agree bit for bit.  Returns (out, lse)."""
+    """Forward under every emulator setting -- moves landing late or at once, workgroups in another
+    order, a workgroup's wavefronts advancing together or one at a time for random stretches;
+    results must agree bit for bit.  Returns (out, lse)."""
     results = []
-    settings = [(False, 0), (True, 0)] + ([(False, 12345), (True, 777)] if n_splits > 1 else [])
-    for eager, order in settings:
-        harness.configure(dma_eager=eager, block_order_seed=order)
+    settings = [(False, 0, 0), (True, 0, 0), (False, 0, 1), (True, 0, 2)] + ([(False, 12345, 3), (True, 777, 0)] if n_splits > 1 else [])
+    for eager, order, skew in settings:
+        harness.configure(dma_eager=eager, block_order_seed=order, wave_skew_seed=skew)
         out, lse, rc = harness.forward(cfg, n_splits=n_splits, **kw)
         assert rc == 0, rc
         results.append((out, lse))
@@ -301,7 +313,7 @@ def test_more_than_one_chunk_of_the_list():
         _check(cfg, out, lse)
 
 
-def test_plumbing_f32_scalar_kernel():
+def test_plumbing_f32_scalar_kernel(schedule):
     from flagtree_amd import workloads
     cfg = workloads.plumbing_f32("cpu", tokens=2, heads=16, s_kv=512, topk=64)
     out, lse, rc = harness.forward(cfg, n_splits=1)
@@ -522,7 +534,7 @@ def _header(ws):
 
 @pytest.mark.parametrize("heads", [128, 16])
 @pytest.mark.parametrize("stale", ["one ticket", "own bit", "all ones"])
-def test_stale_arrival_word_is_flagged_not_hung(heads, stale):
+def test_stale_arrival_word_is_flagged_not_hung(heads, stale, schedule):
     from flagtree_amd import _lib, workloads
     cfg = workloads.decode_bf16("cpu", batch=3, heads=heads, pages_per_seq=6, topk=260, pad_frac=0.05)
     ref_out, ref_lse, rc = harness.forward(cfg, n_splits=1)
@@ -546,7 +558,7 @@ def test_stale_arrival_word_is_flagged_not_hung(heads, stale):
     assert max_abs(to_np(lse2), to_np(ref_lse)) <= 1e-3 and max_abs(to_np(out2), to_np(ref_out)) <= 1e-2
 
 
-def test_uninitialised_workspace_is_flagged():
+def test_uninitialised_workspace_is_flagged(schedule):
     from flagtree_amd import _lib, workloads
     cfg = workloads.decode_bf16("cpu", batch=2, heads=128, pages_per_seq=6, topk=260, pad_frac=0.05)
     ws = torch.zeros(harness.lib().smla_workspace_bytes(2, 128, 512, 2), dtype=torch.uint8)
@@ -559,7 +571,7 @@ def test_uninitialised_workspace_is_flagged():
 
 # ---- integer / byte paths: bit-exact ------------------------------------------------------------
 
-def test_gather_and_translation_bit_exact():
+def test_gather_and_translation_bit_exact(schedule):
     from flagtree_amd import workloads
     cfg = workloads.decode_bf16("cpu", batch=5, heads=16, pages_per_seq=8, topk=96, pad_frac=0.2)
     idx = cfg["indices"].clone().view(5, 96)
@@ -579,7 +591,7 @@ def test_gather_and_translation_bit_exact():
     assert np.array_equal(to_np(rows), oracle.gather_rows(to_np(kv), want))
 
 
-def test_cache_writer_bit_exact():
+def test_cache_writer_bit_exact(schedule):
     g = torch.Generator().manual_seed(3)
     latent = (torch.randn((200, 576), generator=g) * torch.logspace(-3, 2, 200).view(-1, 1)).to(torch.bfloat16)
     latent[5, 100:228] = 0                                   # an all-zero block
@@ -601,10 +613,14 @@ def test_topk_indices_exact(rows, n, k):
     scores[0, : n // 3] = scores[0, 0]                        # ties across the selection boundary
     scores[-1, 5 % n] = float("nan")
     lens = torch.randint(1, n + 1, (rows,), generator=g, dtype=torch.int32)
-    out = torch.full((rows, k), -9, dtype=torch.int32)
-    rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), rows, n, n, k, None)
-    assert rc == 0
-    assert np.array_equal(to_np(out), oracle.topk_indices(to_np(scores), k, to_np(lens)))
+    want = oracle.topk_indices(to_np(scores), k, to_np(lens))
+    for skew in (0, 1, 2):
+        harness.configure(wave_skew_seed=skew)
+        out = torch.full((rows, k), -9, dtype=torch.int32)
+        rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), rows, n, n, k, None)
+        assert rc == 0
+        assert np.array_equal(to_np(out), want), skew
+    harness.configure()
 
 
 @pytest.mark.parametrize("n,length,k", [(65537, 300, 64), (65537, 10117, 300), (70001, 70001, 2048), (65536, 1000, 64)])
@@ -617,10 +633,14 @@ def test_topk_indices_with_tied_values_in_long_rows(n, length, k):
     g = torch.Generator().manual_seed(n + length + k)
     scores = (torch.randn((2, n), generator=g) * 4).round() / 4
     lens = torch.tensor([length, max(1, length // 3)], dtype=torch.int32)
-    out = torch.full((2, k), -9, dtype=torch.int32)
-    rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), 2, n, n, k, None)
-    assert rc == 0
-    assert np.array_equal(to_np(out), oracle.topk_indices(to_np(scores), k, to_np(lens)))
+    want = oracle.topk_indices(to_np(scores), k, to_np(lens))
+    for skew in (0, 1):
+        harness.configure(wave_skew_seed=skew)
+        out = torch.full((2, k), -9, dtype=torch.int32)
+        rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), 2, n, n, k, None)
+        assert rc == 0
+        assert np.array_equal(to_np(out), want), skew
+    harness.configure()
 
 
 @pytest.mark.parametrize("m,n,k,chunks", [(256, 256, 128, 2), (128, 512, 192, 1), (384, 256, 64, 3), (512, 256, 128, 4),
@@ -632,8 +652,8 @@ def test_local_gemm(m, n, k, chunks):
     w = (torch.randn((k, n), generator=g) * 0.1).to(torch.bfloat16)
     partial = torch.randn((m, n), generator=g)
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16)
-    for eager in (False, True):
-        harness.configure(dma_eager=eager)
+    for eager, skew in ((False, 0), (True, 0), (False, 1), (True, 2)):
+        harness.configure(dma_eager=eager, wave_skew_seed=skew)
         rc = harness.lib().smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), partial.data_ptr(), out.data_ptr(), m, n, k, chunks,
                                               (m // chunks) * n, None)
         assert rc == 0
