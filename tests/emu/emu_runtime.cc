@@ -169,10 +169,18 @@ bool run_wave_once(size_t wv) {
 void run_block_skewed(Dim3 bidx) {
   std::mt19937 rng(g_wave_skew * 2654435761u + bidx.x * 40503u + bidx.y * 97u + bidx.z);
   const size_t n_waves = g_block.waves.size();
+  // seeds from 1000 on: one wavefront (seed % wavefronts) is held back -- it only gets a turn, one
+  // step at a time, when none of the others can move
+  const bool hold_one = g_wave_skew >= 1000;
+  const size_t held = g_wave_skew % n_waves;
   unsigned long long stuck_draws = 0;
   while (g_block.live > 0) {
-    const size_t wv = rng() % n_waves;
-    const unsigned stretch = 1u + rng() % ((rng() & 3) == 0 ? 4096u : 48u);      // mostly short, now and then as far as it gets
+    size_t wv = rng() % n_waves;
+    unsigned stretch = 1u + rng() % ((rng() & 3) == 0 ? 4096u : 48u);            // mostly short, now and then as far as it gets
+    if (hold_one) {
+      if (stuck_draws >= 8 * n_waves) { wv = held; stretch = 1; }
+      else if (wv == held) wv = (wv + 1) % n_waves;
+    }
     bool any = false;
     for (unsigned r = 0; r < stretch && run_wave_once(wv); ++r) any = true;
     if (any) {

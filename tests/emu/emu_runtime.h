@@ -79,7 +79,8 @@ extern "C" {
 // knobs for the tests
 void emu_set_dma_mode(int eager);        // 0: moves land at the wait (default), 1: at issue
 void emu_set_block_order(unsigned seed); // 0: ascending block ids, else a seeded shuffle
-void emu_set_wave_skew(unsigned seed);   // 0: a workgroup's wavefronts advance together; else they run one at a time for random stretches
+void emu_set_wave_skew(unsigned seed);   // 0: a workgroup's wavefronts advance together; else they run one at a time for random
+                                         // stretches; from 1000 on wavefront (seed % wavefronts) also moves only when no other can
 unsigned long long emu_launch_count(void);
 void emu_set_cu_count(int n);            // before the library's first query (it caches the answer); default 256
 void emu_set_lds_profile(int on);        // 1: count bank passes of the kernels' addressed LDS accesses (slower); resets the counts

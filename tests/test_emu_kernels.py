@@ -61,7 +61,8 @@ def _forward_all_ways(cfg, n_splits, **kw):
     order, a workgroup's wavefronts advancing together or one at a time for random stretches;
     results must agree bit for bit.  Returns (out, lse)."""
     results = []
-    settings = [(False, 0, 0), (True, 0, 0), (False, 0, 1), (True, 0, 2)] + ([(False, 12345, 3), (True, 777, 0)] if n_splits > 1 else [])
+    # (skew seeds from 1000 on also hold one wavefront back until no other can move)
+    settings = [(False, 0, 0), (True, 0, 0), (False, 0, 1), (True, 0, 1002)] + ([(False, 12345, 3), (True, 777, 1001)] if n_splits > 1 else [])
     for eager, order, skew in settings:
         harness.configure(dma_eager=eager, block_order_seed=order, wave_skew_seed=skew)
         out, lse, rc = harness.forward(cfg, n_splits=n_splits, **kw)
