@@ -14,7 +14,9 @@ from flagtree_amd import _lib as product_lib
 HERE = os.path.dirname(os.path.abspath(__file__))
 _lib = None
 _keep_alive = []
-EMU_CUS = 16      # compute units the stand-in device reports: small, so that small shapes reach the planning corner cases
+# compute units the stand-in device reports: small, so that small shapes reach the planning corner
+# cases (FLAGTREE_EMU_CUS=256 makes the planners choose what they choose on the real device)
+EMU_CUS = int(os.environ.get("FLAGTREE_EMU_CUS", "16"))
 
 
 def lib():
@@ -38,15 +40,19 @@ def lib():
         l.emu_lds_profile.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
         l.emu_work_counts.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.c_int]
         l.emu_set_cu_count(EMU_CUS)                      # before the library's first (cached) query
+        l.emu_set_wave_skew(DEFAULT_WAVE_SKEW)
         _lib = l
     return _lib
 
 
-def configure(dma_eager=False, block_order_seed=0, wave_skew_seed=0):
+DEFAULT_WAVE_SKEW = int(os.environ.get("FLAGTREE_EMU_WAVE_SKEW", "0"))   # schedule of runs that do not choose one (a rehearsal)
+
+
+def configure(dma_eager=False, block_order_seed=0, wave_skew_seed=None):
     l = lib()
     l.emu_set_dma_mode(1 if dma_eager else 0)
     l.emu_set_block_order(block_order_seed)
-    l.emu_set_wave_skew(wave_skew_seed)
+    l.emu_set_wave_skew(DEFAULT_WAVE_SKEW if wave_skew_seed is None else wave_skew_seed)
 
 
 def lds_profile_start():
