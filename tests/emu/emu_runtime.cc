@@ -12,6 +12,7 @@
 
 #include <algorithm>
 #include <random>
+#include <memory>
 #include <vector>
 
 extern "C" char __start_emu_lds[];
@@ -47,6 +48,7 @@ namespace emu {
 namespace {
 
 constexpr size_t kStackBytes = 256 * 1024;
+constexpr unsigned kMaxBlockThreads = 1024;
 
 struct Fiber {
   Lane lane;
@@ -90,9 +92,19 @@ struct Block {
   int live = 0;
   int arrived = 0;
   unsigned long long gen = 0;
+  unsigned long long polls = 0;    // times a lane gave way inside a polling loop (counts as progress)
+  // for workgroups that share the machine (see launch): its id, its LDS while another one runs,
+  // the stacks it uses, the state of its skewed schedule
+  Dim3 idx;
+  std::vector<uint8_t> lds;
+  size_t stack_slot = 0;
+  std::mt19937 rng;
+  unsigned long long stuck_draws = 0, idle_rounds = 0;
 };
 
-Block g_block;
+Block g_solo;
+Block* g_blk = &g_solo;
+#define g_block (*g_blk)
 Fiber* g_cur = nullptr;
 void* g_sched_sp = nullptr;
 Dim3 g_block_idx, g_block_dim, g_grid_dim;
@@ -100,7 +112,10 @@ const std::function<void()>* g_body = nullptr;
 int g_dma_eager = 0;
 unsigned g_order_seed = 0;
 unsigned g_wave_skew = 0;
+unsigned g_concurrent = 0;         // 0 / 1: workgroups run one after the other; n: up to n share the machine
+unsigned g_concurrent_seed = 0;
 unsigned long long g_launches = 0;
+unsigned long long g_polls = 0;
 int g_cu_count = 256;
 std::vector<char*> g_stacks;
 
@@ -166,44 +181,79 @@ bool run_wave_once(size_t wv) {
 // but barriers keeps wavefronts in step; a kernel that relies on them advancing together (a ring
 // slot refilled while a slower wavefront still reads it, a flag read before it is written)
 // passes under the even schedule and fails under this one.
-void run_block_skewed(Dim3 bidx) {
-  std::mt19937 rng(g_wave_skew * 2654435761u + bidx.x * 40503u + bidx.y * 97u + bidx.z);
-  const size_t n_waves = g_block.waves.size();
+// One draw of it, on the current workgroup:
+void step_block_skewed() {
+  Block& b = g_block;
+  const size_t n_waves = b.waves.size();
   // seeds from 1000 on: one wavefront (seed % wavefronts) is held back -- it only gets a turn, one
   // step at a time, when none of the others can move
   const bool hold_one = g_wave_skew >= 1000;
   const size_t held = g_wave_skew % n_waves;
-  unsigned long long stuck_draws = 0;
-  while (g_block.live > 0) {
-    size_t wv = rng() % n_waves;
-    unsigned stretch = 1u + rng() % ((rng() & 3) == 0 ? 4096u : 48u);            // mostly short, now and then as far as it gets
-    if (hold_one) {
-      if (stuck_draws >= 8 * n_waves) { wv = held; stretch = 1; }
-      else if (wv == held) wv = (wv + 1) % n_waves;
-    }
-    bool any = false;
-    for (unsigned r = 0; r < stretch && run_wave_once(wv); ++r) any = true;
-    if (any) {
-      stuck_draws = 0;
-    } else if (++stuck_draws > 64 * n_waves) {                                   // every wavefront drawn many times, none could run
-      fail("deadlock in block (%u,%u,%u): %d lanes wait at barriers that cannot complete", bidx.x, bidx.y, bidx.z, g_block.live);
-    }
+  size_t wv = b.rng() % n_waves;
+  unsigned stretch = 1u + b.rng() % ((b.rng() & 3) == 0 ? 4096u : 48u);          // mostly short, now and then as far as it gets
+  if (hold_one) {
+    if (b.stuck_draws >= 8 * n_waves) { wv = held; stretch = 1; }
+    else if (wv == held) wv = (wv + 1) % n_waves;
+  }
+  bool any = false;
+  for (unsigned r = 0; r < stretch && run_wave_once(wv); ++r) any = true;
+  if (any) {
+    b.stuck_draws = 0;
+  } else if (++b.stuck_draws > 64 * n_waves) {                                   // every wavefront drawn many times, none could run
+    fail("deadlock in block (%u,%u,%u): %d lanes wait at barriers that cannot complete", b.idx.x, b.idx.y, b.idx.z, b.live);
   }
 }
 
-void run_block(Dim3 bidx) {
+// Even schedule, one round: every lane that can run does, up to its next rendezvous.  A full round
+// without any lane finishing, any rendezvous completing or any polling loop giving way means the
+// lanes are waiting for each other in different places.
+void step_block_even() {
+  Block& b = g_block;
+  unsigned long long before = b.gen + b.polls;
+  for (Wave& w : b.waves) before += w.gen;
+  const int live_before = b.live;
+  for (Fiber& f : b.fibers) {
+    if (f.done) continue;
+    if (f.wait_gen != nullptr && *f.wait_gen == f.wait_val) continue;
+    f.wait_gen = nullptr;
+    g_cur = &f;
+    emu_switch(&g_sched_sp, f.sp);
+  }
+  unsigned long long after = b.gen + b.polls;
+  for (Wave& w : b.waves) after += w.gen;
+  if (after == before && b.live == live_before) {
+    if (++b.idle_rounds > 4)
+      fail("deadlock in block (%u,%u,%u): %d lanes wait at barriers that cannot complete", b.idx.x, b.idx.y, b.idx.z, b.live);
+  } else {
+    b.idle_rounds = 0;
+  }
+}
+
+void step_block() {
+  if (g_wave_skew != 0 && g_block.waves.size() > 1) step_block_skewed();
+  else step_block_even();
+  g_cur = nullptr;
+}
+
+// Makes `b` the current workgroup, with all its lanes at the start of the kernel.  Does not touch LDS.
+void setup_block(Block& b, Dim3 bidx, size_t stack_slot) {
   const unsigned n = g_block_dim.x * g_block_dim.y * g_block_dim.z;
   const unsigned n_waves = (n + kWave - 1) / kWave;
+  if (n > kMaxBlockThreads) fail("workgroup of %u lanes", n);
+  g_blk = &b;
   g_block_idx = bidx;
-  g_block.fibers.assign(n, Fiber());
-  g_block.waves.assign(n_waves, Wave());
-  g_block.live = (int)n;
-  g_block.arrived = 0;
-  g_block.gen = 0;
-  memset(__start_emu_lds, 0xFB, __stop_emu_lds - __start_emu_lds);   // LDS holds no defined values at workgroup start
+  b.idx = bidx;
+  b.stack_slot = stack_slot;
+  b.rng.seed(g_wave_skew * 2654435761u + bidx.x * 40503u + bidx.y * 97u + bidx.z);
+  b.stuck_draws = b.idle_rounds = b.polls = 0;
+  b.fibers.assign(n, Fiber());
+  b.waves.assign(n_waves, Wave());
+  b.live = (int)n;
+  b.arrived = 0;
+  b.gen = 0;
   for (unsigned i = 0; i < n; ++i) {
-    Fiber& f = g_block.fibers[i];
-    Wave& w = g_block.waves[i / kWave];
+    Fiber& f = b.fibers[i];
+    Wave& w = b.waves[i / kWave];
     f.lane.flat = (int)i;
     f.lane.lane = (int)(i % kWave);
     f.lane.tid = Dim3(i % g_block_dim.x, (i / g_block_dim.x) % g_block_dim.y, i / (g_block_dim.x * g_block_dim.y));
@@ -211,42 +261,62 @@ void run_block(Dim3 bidx) {
     w.n_lanes++;
     w.live++;
     w.lane_live[i % kWave] = true;
-    f.stack = get_stack(i);
+    f.stack = get_stack(stack_slot * kMaxBlockThreads + i);
     prepare(&f);
   }
-  for (Wave& w : g_block.waves) {
+  for (Wave& w : b.waves) {
     for (int l = w.n_lanes; l < kWave; ++l) w.lane_live[l] = false;
     w.took_part[0] = w.took_part[1] = w.n_lanes == kWave ? ~0ull : (1ull << w.n_lanes) - 1ull;
   }
-  if (g_wave_skew != 0 && n_waves > 1) {
-    run_block_skewed(bidx);
-    g_cur = nullptr;
-    return;
-  }
-  // round-robin until every lane has left; a full round without any lane finishing or any
-  // rendezvous completing means the lanes are waiting for each other in different places
-  unsigned long long idle_rounds = 0;
-  while (g_block.live > 0) {
-    unsigned long long before = g_block.gen;
-    for (Wave& w : g_block.waves) before += w.gen;
-    const int live_before = g_block.live;
-    for (Fiber& f : g_block.fibers) {
-      if (f.done) continue;
-      if (f.wait_gen != nullptr && *f.wait_gen == f.wait_val) continue;
-      f.wait_gen = nullptr;
-      g_cur = &f;
-      emu_switch(&g_sched_sp, f.sp);
+}
+
+// One workgroup from start to end, alone on the machine.
+void run_block(Dim3 bidx) {
+  setup_block(g_solo, bidx, 0);
+  memset(__start_emu_lds, 0xFB, __stop_emu_lds - __start_emu_lds);   // LDS holds no defined values at workgroup start
+  while (g_block.live > 0) step_block();
+}
+
+// Up to `g_concurrent` workgroups share the machine: one of them, drawn at random, advances by a
+// few scheduling steps, then another.  The one LDS arena holds the running workgroup's contents;
+// the others' are kept aside.  What this adds over one workgroup at a time: a workgroup that waits
+// for another one (the last arrival of a split merge polling for the others' published bits)
+// really waits, and the others really publish while it does.
+void run_blocks_concurrently(const std::vector<size_t>& order, Dim3 grid) {
+  const size_t lds_size = (size_t)(__stop_emu_lds - __start_emu_lds);
+  std::mt19937 rng(g_concurrent_seed * 7919u + 13u);
+  std::vector<std::unique_ptr<Block>> active;
+  std::vector<size_t> free_slots;
+  for (size_t k = g_concurrent; k-- > 0;) free_slots.push_back(k);
+  size_t next = 0;
+  Block* in_lds = nullptr;
+  while (next < order.size() || !active.empty()) {
+    while (active.size() < g_concurrent && next < order.size()) {
+      const size_t i = order[next++];
+      active.emplace_back(new Block());
+      active.back()->lds.assign(lds_size, 0xFB);
+      setup_block(*active.back(), Dim3((unsigned)(i % grid.x), (unsigned)((i / grid.x) % grid.y), (unsigned)(i / ((size_t)grid.x * grid.y))),
+                  free_slots.back());
+      free_slots.pop_back();
     }
-    unsigned long long after = g_block.gen;
-    for (Wave& w : g_block.waves) after += w.gen;
-    if (after == before && g_block.live == live_before) {
-      if (++idle_rounds > 4)
-        fail("deadlock in block (%u,%u,%u): %d lanes wait at barriers that cannot complete", bidx.x, bidx.y, bidx.z, g_block.live);
-    } else {
-      idle_rounds = 0;
+    const size_t pick = rng() % active.size();
+    Block* b = active[pick].get();
+    if (in_lds != b) {
+      if (in_lds != nullptr) memcpy(in_lds->lds.data(), __start_emu_lds, lds_size);
+      memcpy(__start_emu_lds, b->lds.data(), lds_size);
+      in_lds = b;
+    }
+    g_blk = b;
+    g_block_idx = b->idx;
+    const unsigned quanta = 1u + rng() % 8u;
+    for (unsigned q = 0; q < quanta && b->live > 0; ++q) step_block();
+    if (b->live == 0) {
+      free_slots.push_back(b->stack_slot);
+      in_lds = nullptr;
+      active.erase(active.begin() + (long)pick);
     }
   }
-  g_cur = nullptr;
+  g_blk = &g_solo;
 }
 
 }  // namespace
@@ -294,6 +364,12 @@ int wave_rendezvous(const void* post, size_t bytes, uint32_t tag) {
 
 const uint8_t* wave_slot(int parity, int lane) { return g_cur->lane.wave->slot[parity][lane]; }
 bool wave_lane_live(int lane) { return (g_cur->lane.wave->took_part[g_cur->lane.parity] >> lane) & 1; }
+
+void poll_yield() {
+  g_block.polls++;
+  g_polls++;
+  yield();
+}
 
 void block_barrier() {
   g_work.barriers_lane_calls++;
@@ -449,8 +525,13 @@ void launch(Dim3 grid, Dim3 block, const std::function<void()>& body) {
     std::mt19937 rng(g_order_seed);
     std::shuffle(order.begin(), order.end(), rng);
   }
-  for (size_t i : order)
-    run_block(Dim3((unsigned)(i % grid.x), (unsigned)((i / grid.x) % grid.y), (unsigned)(i / ((size_t)grid.x * grid.y))));
+  if (g_concurrent > 1 && n_blocks > 1) {
+    run_blocks_concurrently(order, grid);
+  } else {
+    for (size_t i : order)
+      run_block(Dim3((unsigned)(i % grid.x), (unsigned)((i / grid.x) % grid.y), (unsigned)(i / ((size_t)grid.x * grid.y))));
+  }
+  g_cur = nullptr;
   g_body = nullptr;
 }
 
@@ -460,7 +541,9 @@ extern "C" {
 void emu_set_dma_mode(int eager) { emu::g_dma_eager = eager; }
 void emu_set_block_order(unsigned seed) { emu::g_order_seed = seed; }
 void emu_set_wave_skew(unsigned seed) { emu::g_wave_skew = seed; }
+void emu_set_concurrent_blocks(unsigned n, unsigned seed) { emu::g_concurrent = n; emu::g_concurrent_seed = seed; }
 unsigned long long emu_launch_count(void) { return emu::g_launches; }
+unsigned long long emu_poll_count(void) { return emu::g_polls; }
 void emu_set_cu_count(int n) { emu::g_cu_count = n; }
 void emu_set_lds_profile(int on) {
   emu::g_lds_profile = on != 0;

@@ -47,6 +47,7 @@ int wave_rendezvous(const void* post, size_t bytes, uint32_t tag);
 const uint8_t* wave_slot(int parity, int lane);      // what `lane` posted (valid until the next rendezvous but one)
 bool wave_lane_live(int lane);                       // `lane` took part in the calling lane's last rendezvous
 void block_barrier();
+void poll_yield();                                   // inside a loop that polls memory another workgroup writes: lets the others run
 
 // LDS arena: every __shared__ object lives in the ELF section "emu_lds"
 uint32_t lds_addr(const void* p);
@@ -81,7 +82,11 @@ void emu_set_dma_mode(int eager);        // 0: moves land at the wait (default),
 void emu_set_block_order(unsigned seed); // 0: ascending block ids, else a seeded shuffle
 void emu_set_wave_skew(unsigned seed);   // 0: a workgroup's wavefronts advance together; else they run one at a time for random
                                          // stretches; from 1000 on wavefront (seed % wavefronts) also moves only when no other can
+// n > 1: up to n workgroups share the machine, each advancing a few scheduling steps at a time in a seeded random order
+// (a workgroup that polls for another one's writes then really waits); else one workgroup after the other
+void emu_set_concurrent_blocks(unsigned n, unsigned seed);
 unsigned long long emu_launch_count(void);
+unsigned long long emu_poll_count(void);  // times a lane gave way inside a polling loop since the library was loaded
 void emu_set_cu_count(int n);            // before the library's first query (it caches the answer); default 256
 void emu_set_lds_profile(int on);        // 1: count bank passes of the kernels' addressed LDS accesses (slower); resets the counts
 // out[3 * kind + 0] wavefront instructions, + 1 passes they took, + 2 passes a conflict-free access would take

@@ -34,7 +34,9 @@ def lib():
         l.emu_set_dma_mode.argtypes = [ctypes.c_int]
         l.emu_set_block_order.argtypes = [ctypes.c_uint]
         l.emu_set_wave_skew.argtypes = [ctypes.c_uint]
+        l.emu_set_concurrent_blocks.argtypes = [ctypes.c_uint, ctypes.c_uint]
         l.emu_launch_count.restype = ctypes.c_ulonglong
+        l.emu_poll_count.restype = ctypes.c_ulonglong
         l.emu_set_cu_count.argtypes = [ctypes.c_int]
         l.emu_set_lds_profile.argtypes = [ctypes.c_int]
         l.emu_lds_profile.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
@@ -48,8 +50,9 @@ def lib():
 DEFAULT_WAVE_SKEW = int(os.environ.get("FLAGTREE_EMU_WAVE_SKEW", "0"))   # schedule of runs that do not choose one (a rehearsal)
 
 
-def configure(dma_eager=False, block_order_seed=0, wave_skew_seed=None):
+def configure(dma_eager=False, block_order_seed=0, wave_skew_seed=None, concurrent_blocks=0, concurrent_seed=0):
     l = lib()
+    l.emu_set_concurrent_blocks(concurrent_blocks, concurrent_seed)
     l.emu_set_dma_mode(1 if dma_eager else 0)
     l.emu_set_block_order(block_order_seed)
     l.emu_set_wave_skew(DEFAULT_WAVE_SKEW if wave_skew_seed is None else wave_skew_seed)

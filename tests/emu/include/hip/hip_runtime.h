@@ -92,7 +92,7 @@ inline int __ffsll(long long v) { return __builtin_ffsll(v); }
 inline void __syncthreads() { emu::block_barrier(); }
 #define __builtin_amdgcn_sched_barrier(m) ((void)0)
 #define __builtin_amdgcn_sched_group_barrier(a, b, c) ((void)0)
-#define __builtin_amdgcn_s_sleep(n) ((void)0)
+#define __builtin_amdgcn_s_sleep(n) emu::poll_yield()   /* the kernels sleep only inside loops that poll another workgroup's writes */
 #define __builtin_amdgcn_s_setprio(n) ((void)0)
 #define __builtin_amdgcn_wave_barrier() ((void)emu::wave_rendezvous(nullptr, 0, 0x57415645u))
 

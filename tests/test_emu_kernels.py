@@ -58,13 +58,15 @@ def _check(cfg, out, lse, out_tol=OUT_TOL, lse_tol=LSE_TOL):
 
 def _forward_all_ways(cfg, n_splits, **kw):
     """Forward under every emulator setting -- moves landing late or at once, workgroups in another
-    order, a workgroup's wavefronts advancing together or one at a time for random stretches;
-    results must agree bit for bit.  Returns (out, lse)."""
+    order, one after the other or several sharing the machine, a workgroup's wavefronts advancing
+    together or one at a time for random stretches; results must agree bit for bit.  Returns (out, lse)."""
     results = []
-    # (skew seeds from 1000 on also hold one wavefront back until no other can move)
-    settings = [(False, 0, 0), (True, 0, 0), (False, 0, 1), (True, 0, 1002)] + ([(False, 12345, 3), (True, 777, 1001)] if n_splits > 1 else [])
-    for eager, order, skew in settings:
-        harness.configure(dma_eager=eager, block_order_seed=order, wave_skew_seed=skew)
+    # (skew seeds from 1000 on also hold one wavefront back until no other can move; the last number:
+    # how many workgroups share the machine -- with splits, so that the merging one has to wait)
+    settings = [(False, 0, 0, 0), (True, 0, 0, 0), (False, 0, 1, 0), (True, 0, 1002, 0)] + (
+        [(False, 12345, 5, 4), (True, 777, 1001, 0), (True, 5, 0, 16)] if n_splits > 1 else [])
+    for eager, order, skew, together in settings:
+        harness.configure(dma_eager=eager, block_order_seed=order, wave_skew_seed=skew, concurrent_blocks=together, concurrent_seed=order)
         out, lse, rc = harness.forward(cfg, n_splits=n_splits, **kw)
         assert rc == 0, rc
         results.append((out, lse))
@@ -531,6 +533,39 @@ def _words(ws):
 def _header(ws):
     from flagtree_amd import _lib
     return ws[_lib.SMLA_WS_HEADER_OFFSET:_lib.SMLA_WS_HEADER_OFFSET + 16].view(torch.int32)
+
+
+@pytest.mark.parametrize("kernel", ["many_heads", "eight_wavefronts", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split"])
+def test_merging_workgroup_really_waits_for_the_others(kernel, monkeypatch):
+    """With one workgroup at a time the last arrival of a split merge always finds the others'
+    partials published.  Here several share the machine and are switched every few steps: the
+    merging workgroup polls, the others publish meanwhile (the poll count says it happened), and
+    the results are the same bits as without any waiting."""
+    from flagtree_amd import workloads
+    heads = 128 if kernel in ("many_heads", "eight_wavefronts", "wavefront_per_head_group") else 16
+    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", {"eight_wavefronts": "1", "wavefront_per_head_group": "2"}.get(kernel, "0"))
+    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel == "few_heads_fp8_column_split" else "0")
+    if kernel == "few_heads_fp8_column_split":
+        cfg, _ = _fp8_cfg(3, heads, 20, 400, pad_frac=0.05)
+    else:
+        cfg = workloads.decode_bf16("cpu", batch=3, heads=heads, pages_per_seq=20, topk=400, pad_frac=0.05)
+    harness.configure()
+    out0, lse0, rc = harness.forward(cfg, n_splits=3)
+    assert rc == 0
+    waited = 0
+    for n, seed in enumerate(range(2, 26)):
+        if n >= 4 and waited > 0:
+            break
+        together, skew = ((4, 5), (16, 0), (6, 9), (3, 5))[n % 4]
+        harness.configure(dma_eager=bool(seed & 1), wave_skew_seed=skew, concurrent_blocks=together, concurrent_seed=seed, block_order_seed=seed)
+        before = harness.lib().emu_poll_count()
+        out, lse, rc = harness.forward(cfg, n_splits=3)
+        waited += harness.lib().emu_poll_count() - before
+        assert rc == 0
+        assert torch.equal(out.view(torch.int16), out0.view(torch.int16)) and torch.equal(lse, lse0)
+    harness.configure()
+    assert waited > 0
+    _check(cfg, out0, lse0)
 
 
 @pytest.mark.parametrize("heads", [128, 16])
