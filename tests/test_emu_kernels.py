@@ -37,12 +37,12 @@ def _emulator():
     harness.configure()
 
 
-@pytest.fixture(params=[0, 3], ids=["wavefronts_in_step", "wavefronts_skewed"])
+@pytest.fixture(params=[(0, 0), (3, 0), (5, 4)], ids=["wavefronts_in_step", "wavefronts_skewed", "workgroups_sharing_the_machine"])
 def schedule(request):
     """For tests that make a single call: once with a workgroup's wavefronts advancing together,
     once with them running one at a time for random stretches (only barriers keep them in step on
-    the hardware)."""
-    harness.configure(wave_skew_seed=request.param)
+    the hardware), once with that and four workgroups at a time switched every few steps."""
+    harness.configure(wave_skew_seed=request.param[0], concurrent_blocks=request.param[1], concurrent_seed=7)
     yield
     harness.configure()
 
