@@ -26,17 +26,37 @@ def _stale(outputs, inputs):
     return any(os.path.getmtime(o) < newest for o in outputs)
 
 
+STAMP_PATH = LIB_PATH + ".stamp"
+
+
+def _digest(paths):
+    """Hash of everything the library is made from (contents, not time stamps: a copy of the tree
+    to another machine keeps the contents)."""
+    import hashlib
+    h = hashlib.sha256(" ".join([CXX] + FLAGS).replace(ROOT, "").encode())
+    for p in sorted(paths):
+        h.update(os.path.relpath(p, ROOT).encode())
+        with open(p, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def build(verbose=False, force=False):
     # every header a kernel source may include (the product's own smla_hw.h is shadowed by the emulator's)
     headers = [os.path.join(HERE, "emu_runtime.h"), os.path.join(HERE, "include", "smla_hw.h"),
                os.path.join(HERE, "include", "hip", "hip_runtime.h"), os.path.join(ROOT, "include", "flagtree_smla.h"),
-               os.path.abspath(__file__)]
+               os.path.abspath(__file__), os.path.join(HW_MODEL, "primitives.h")]
     headers += sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h") and f != "smla_hw.h")
+    names = SOURCES + ["primitives.hip", "emu_runtime.cc"]
+    paths = [os.path.join(HERE if n.endswith(".cc") else (HW_MODEL if n == "primitives.hip" else CSRC), n) for n in names]
+    digest = _digest(paths + headers)
+    # a library that was built from exactly these files is used as it is, also where the object
+    # files did not travel with it (a GPU box runs what was built beforehand and compiles nothing)
+    if not force and os.path.exists(LIB_PATH) and os.path.exists(STAMP_PATH) and open(STAMP_PATH).read().strip() == digest:
+        return LIB_PATH
     objs = []
     procs = []
-    headers.append(os.path.join(HW_MODEL, "primitives.h"))
-    for src in SOURCES + ["primitives.hip", "emu_runtime.cc"]:
-        path = os.path.join(HERE if src.endswith(".cc") else (HW_MODEL if src == "primitives.hip" else CSRC), src)
+    for src, path in zip(names, paths):
         obj = os.path.join(HERE, "build", src + ".o")
         objs.append(obj)
         if not force and not _stale([obj], [path] + headers):
@@ -57,6 +77,8 @@ def build(verbose=False, force=False):
                              stderr=subprocess.STDOUT, text=True)
         if res.returncode != 0:
             raise RuntimeError("emulator link failed:\n" + res.stdout[-4000:])
+    with open(STAMP_PATH, "w") as f:
+        f.write(digest + "\n")
     return LIB_PATH
 
 

@@ -48,7 +48,6 @@ def test_a_wrong_answer_is_noticed():
 
 
 def test_the_gfx950_build_of_the_probes_exports_its_entry_points():
-    import ctypes
     if not os.path.exists(cases.GPU_LIB_PATH):
         pytest.skip("tests/hw_model/libhw_model.so not built")
     with open(cases.GPU_LIB_PATH, "rb") as f:
