@@ -43,9 +43,9 @@ def parse():
                     help="first run three plain 1 GiB device copies (known HBM traffic) so a rocprofv3 --pmc "
                          "run of this command holds a reference kernel to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
-    ap.add_argument("--wide", type=int, nargs="?", const=1, default=0, choices=[0, 1, 2],
-                    help="bf16 many-heads workloads on a 128-heads-per-workgroup kernel (sets FLAGTREE_SMLA_WIDE; 1: eight wavefronts, "
-                         "2: a wavefront per 32 heads; opt-in until measured)")
+    ap.add_argument("--head-groups", action="store_true",
+                    help="many-heads workloads on the 128-heads-per-workgroup kernel, a wavefront per 32 heads (sets "
+                         "FLAGTREE_SMLA_HEAD_GROUPS=1; opt-in until measured)")
     ap.add_argument("--few-fp8", action="store_true",
                     help="decode_fp8 on the two-workgroups-per-CU kernel (sets FLAGTREE_SMLA_FEW_FP8=1; opt-in until measured)")
     ap.add_argument("--token-bands", action="store_true",
@@ -54,11 +54,23 @@ def parse():
     return ap.parse_args()
 
 
+def cpu_threads():
+    """Threads the CPU baseline really runs on: those of the BLAS pool numpy's matrix products use
+    (the environment caps it below what os.cpu_count() shows on a shared box)."""
+    try:
+        import numpy  # noqa: F401  (loads the BLAS library the pool belongs to)
+        from threadpoolctl import threadpool_info
+        n = max((p.get("num_threads", 0) for p in threadpool_info() if p.get("user_api") == "blas"), default=0)
+        if n:
+            return int(n)
+    except Exception:
+        pass
+    return int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count())
+
+
 def many_heads_kernel(a, fmt):
     """Name of the kernel a launch with more than 32 heads goes to under this run's switches."""
-    if a.wide == 2 or (a.wide == 1 and fmt == "bf16"):
-        return {1: "fwd_wide_kernel", 2: "fwd_group_kernel"}[a.wide]
-    return "fwd_tall_kernel"
+    return "fwd_group_kernel" if a.head_groups else "fwd_tall_kernel"
 
 
 def measured_traffic(workload):
@@ -126,8 +138,8 @@ def main():
         sys.exit(2)
     if a.few_fp8:
         os.environ["FLAGTREE_SMLA_FEW_FP8"] = "1"
-    if a.wide:
-        os.environ["FLAGTREE_SMLA_WIDE"] = str(a.wide)
+    if a.head_groups:
+        os.environ["FLAGTREE_SMLA_HEAD_GROUPS"] = "1"
     if a.token_bands:
         os.environ["FLAGTREE_SMLA_TOKEN_BANDS"] = "1"
     import torch
@@ -202,8 +214,9 @@ def main():
     for i in range(a.warmup):
         step(i)
     torch.cuda.synchronize()
-    # The forward is a single kernel launch (the split merge happens inside it), issued on
-    # torch's current stream.  One HIP event pair on that stream brackets the K launches: the
+    # The forward is a single kernel launch (the split merge happens inside it; on a device whose
+    # XCD layout the library does not know, a merge launch follows it), issued on torch's current
+    # stream.  One HIP event pair on that stream brackets the K launches: the
     # span divided by K is the average launch duration including the gap between back-to-back
     # launches; a second pass with one event pair per launch gives the per-launch distribution.
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -237,6 +250,16 @@ def main():
         f1.record()
         torch.cuda.synchronize()
         tail_ms = f0.elapsed_time(f1) / a.steps
+    # A split merge that gave up marks its rows with a NaN LSE and flags the workspace, and every
+    # later launch on that workspace gives up too: no figure is printed for such a run.
+    if ws is not None:
+        ft.workspace_status(ws)                       # raises when any launch above flagged it
+    last_lse = step(0)[1]
+    torch.cuda.synchronize()
+    if not bool(torch.isfinite(last_lse).all().item()):
+        raise RuntimeError("non-finite LSE after the timed loop: the run measured a launch that did not compute")
+    if ws is not None:
+        ft.workspace_status(ws)
 
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     gbs = nbytes / (ms_per_step * 1e-3) / 1e9
@@ -249,7 +272,7 @@ def main():
         roof = dict(bound="mfma", achieved=flops / (kern_ms * 1e-3) / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
     # (the stored counter figures were taken on the default kernels: none for a kernel behind a switch)
-    roof["traffic"] = None if (a.wide or a.few_fp8 or a.token_bands) else measured_traffic(a.workload)
+    roof["traffic"] = None if (a.head_groups or a.few_fp8 or a.token_bands) else measured_traffic(a.workload)
     roof["traffic_source"] = TRAFFIC_NOTE
     roof["kernel"] = many_heads_kernel(a, fmt) if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
     roof["kernel_ms"] = kern_ms
@@ -286,22 +309,22 @@ def main():
     if not a.no_cpu_baseline and a.workload == "prefill_causal_bf16":
         try:
             v, reps, n_rows = cpu_baseline_prefill(cfg)
-            res["cpu_baseline"] = {"value": v, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+            res["cpu_baseline"] = {"value": v, "unit": "TFLOP/s", "cores": cpu_threads(), "kind": "port",
                                    "sample": f"numpy fp32 oracle on a stratified sample of {n_rows} of the {cfg['q'].shape[1]} query "
                                              f"tokens (every {cfg['q'].shape[1] // n_rows}th), median of {reps} runs; a rate, not extrapolated"}
         except Exception as e:
-            res["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+            res["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": cpu_threads(), "kind": "port",
                                    "sample": f"failed: {e}"}
     if not a.no_cpu_baseline and a.workload != "prefill_causal_bf16":
         n_seq = a.cpu_sample or min(cfg["q"].shape[0], 8)
         try:
             import numpy  # noqa: F401
             v, reps = cpu_baseline(cfg, n_seq)
-            res["cpu_baseline"] = {"value": v, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+            res["cpu_baseline"] = {"value": v, "unit": "TFLOP/s", "cores": cpu_threads(), "kind": "port",
                                    "sample": f"numpy fp32 oracle on the first {n_seq} of {cfg['q'].shape[0]} sequences "
                                              f"of the same workload, median of {reps} runs"}
         except Exception as e:   # the baseline is a reported extra; never lose the GPU number over it
-            res["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+            res["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": cpu_threads(), "kind": "port",
                                    "sample": f"failed: {e}"}
     print(json.dumps(res))
 
@@ -346,7 +369,7 @@ def bench_gemm(a, torch, ft, workloads, dev):
         t0 = time.perf_counter()
         oracle.gemm_rs_local(xs, ws, ps, n_chunks=2)
         dt = time.perf_counter() - t0
-        res["cpu_baseline"] = {"value": 2.0 * rows * N * Kd / dt / 1e12, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+        res["cpu_baseline"] = {"value": 2.0 * rows * N * Kd / dt / 1e12, "unit": "TFLOP/s", "cores": cpu_threads(), "kind": "port",
                                "sample": f"numpy oracle (float64, BLAS threads) on the first {rows} of the {M} rows"}
     print(json.dumps(res))
 
@@ -434,7 +457,7 @@ def bench_dense(a, torch, ft, workloads, dev):
         "config": {"workload": "decode_dense_bf16", "batch": B, "heads": H, "context": ctx, "page_size": cfg["page_size"],
                    "flops_per_step": flops, "bytes_per_step": nbytes},
         "roofline": {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": ach / PEAK_BF16_TFLOPS, "traffic": None if a.wide else measured_traffic("decode_dense_bf16"),
+                     "frac": ach / PEAK_BF16_TFLOPS, "traffic": None if a.head_groups else measured_traffic("decode_dense_bf16"),
                      "traffic_source": TRAFFIC_NOTE, "kernel": many_heads_kernel(a, "bf16"), "kernel_ms": kern_ms,
                      "other_bound": {"bound": "hbm", "achieved": nbytes / (kern_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                                      "unit": "GB/s", "frac": nbytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}},
@@ -448,11 +471,11 @@ def bench_dense(a, torch, ft, workloads, dev):
             from _util import oracle_inputs
             qn, kv_small, phys_small, _ = oracle_inputs(sub)
             v, reps = _time_oracle(qn, kv_small, phys_small, cfg["sm_scale"])
-            res["cpu_baseline"] = {"value": v, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+            res["cpu_baseline"] = {"value": v, "unit": "TFLOP/s", "cores": cpu_threads(), "kind": "port",
                                    "sample": f"numpy fp32 oracle on the first {n_seq} of {B} sequences of the same workload, "
                                              f"median of {reps} runs"}
         except Exception as e:
-            res["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+            res["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": cpu_threads(), "kind": "port",
                                    "sample": f"failed: {e}"}
     print(json.dumps(res))
 

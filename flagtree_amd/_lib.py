@@ -27,6 +27,7 @@ SIGNATURES = {
     "smla_fwd_scalar": (_c.c_int, [_c.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
                                    _i32, _i32, _i32, _i64, _i64, _f32, _vp]),
     "smla_plan_splits": (_c.c_int, [_c.c_int, _i32, _i32, _i32]),
+    "smla_merge_in_launch": (_c.c_int, []),
     "smla_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
     "smla_workspace_init": (_c.c_int, [_vp, _sz, _vp]),
     "smla_workspace_status": (_c.c_int, [_vp, _sz, _vp, _c.POINTER(_c.c_uint32)]),
@@ -47,7 +48,7 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
-    path = os.environ.get("FLAGTREE_SMLA_LIB", LIB_PATH)     # override: load another build of the same ABI
+    path = LIB_PATH
     if not os.path.exists(path):
         raise RuntimeError(
             f"{path} is missing: build it with `python -m flagtree_amd.build` "

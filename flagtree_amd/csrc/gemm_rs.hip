@@ -417,9 +417,11 @@ void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
 // 896 tiles on 256 units are 3 rounds + 128 tiles, which as 256 half tiles keep every unit busy for
 // 3/4 of a round (a half tile moves 3/4 of a tile's bytes into LDS) instead of half the units for a
 // whole one.
+// The kernel's half-tile mapping takes whole tiles in groups of 8 (one per XCD), so the count
+// of whole tiles must be a multiple of 8: only a compute-unit count that is one gives that.
 int gemm_full_tiles(int mt, int nt, int n_cu) {
   const long long tiles = (long long)mt * nt;
-  if (mt % 8 != 0 || n_cu <= 0) return (int)tiles;
+  if (mt % 8 != 0 || n_cu <= 0 || n_cu % 8 != 0) return (int)tiles;
   const long long rest = tiles % n_cu;
   return rest > 0 && 2 * rest <= n_cu ? (int)(tiles - rest) : (int)tiles;
 }

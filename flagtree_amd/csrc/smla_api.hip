@@ -28,13 +28,12 @@ int check_common(const void* q, const void* kv, const int32_t* indices, const vo
 // Kernels that have passed the parity checks but whose speed has not been measured on hardware
 // yet stay behind a switch until it has (read at every call): FLAGTREE_SMLA_FEW_FP8=1 sends few-heads launches over an
 // fp8 cache to the two-workgroups-per-CU kernel (smla_mfma_few_fp8.hip).  Read at every call.
-// FLAGTREE_SMLA_WIDE=1 or 2 sends many-heads launches to a 128-heads-per-workgroup kernel: 1 = eight
-// wavefronts (smla_mfma_wide.hip, bf16 cache only), 2 = a wavefront per 32 heads (smla_mfma_group.hip).
-int wide_mode() {                            // 0: off
-  const char* e = getenv("FLAGTREE_SMLA_WIDE");
-  return e == nullptr ? 0 : (e[0] == '1' ? 1 : (e[0] == '2' ? 2 : 0));
+// FLAGTREE_SMLA_HEAD_GROUPS=1 sends many-heads launches (either cache format) to the kernel that
+// takes 128 heads per workgroup, a wavefront per 32 heads (smla_mfma_group.hip).
+bool head_groups_enabled() {
+  const char* e = getenv("FLAGTREE_SMLA_HEAD_GROUPS");
+  return e != nullptr && e[0] == '1';
 }
-bool wide_enabled() { return wide_mode() != 0; }
 
 bool few_fp8_enabled() {
   const char* e = getenv("FLAGTREE_SMLA_FEW_FP8");
@@ -48,17 +47,31 @@ bool token_bands_enabled() {
   return e != nullptr && e[0] == '1';
 }
 
+// Compute units of the current device (256 when there is none to ask: planning calls made on a
+// machine without a GPU).  Asked at every call: the answer belongs to the device that is current
+// now, the query is a table look-up in the runtime, and a cache would have to be keyed by device
+// and guarded against concurrent callers for no measurable gain.
 int device_cus() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      cus = n;
-    else
-      return 256;
-  }
-  return cus;
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) == hipSuccess &&
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+    return n;
+  return 256;
+}
+
+// The merge inside the launch passes partials between workgroups through the L2 without fences,
+// which is only correct when every workgroup of a token runs behind the same L2.  The kernels
+// give those workgroups block ids 8 apart; the hardware deals block ids round-robin to the XCDs of
+// the device, so ids 8 apart share an XCD whenever the XCD count divides 8.  On gfx950 an XCD has
+// 32 compute units and a device (a whole GPU or a partition of it) has 1, 2, 4 or 8 of them; any
+// other compute-unit count is a layout this code knows nothing about, and there, or when
+// FLAGTREE_SMLA_SEPARATE_MERGE=1 asks for it, every split publishes its partial and a second
+// launch merges them (a kernel boundary makes the partials visible everywhere).
+bool merge_in_launch_ok() {
+  const char* e = getenv("FLAGTREE_SMLA_SEPARATE_MERGE");
+  if (e != nullptr && e[0] == '1') return false;
+  const int n = device_cus();
+  return n <= 32 || n == 64 || n == 128 || n == 256;
 }
 
 }  // namespace
@@ -82,7 +95,9 @@ const char* smla_strerror(int status) {
   return "unknown status";
 }
 
-int smla_abi_version(void) { return 2; }
+int smla_abi_version(void) { return 3; }
+
+int smla_merge_in_launch(void) { return merge_in_launch_ok() ? 1 : 0; }
 
 // Workspace layout: [0, SMLA_WS_HEADER_OFFSET) arrival words (zero between calls), the 64-byte
 // header {magic, status, poll limit, -} up to SMLA_WS_COUNTER_BYTES, then the partial outputs [T, n_splits, H, d_v] f32 and the partial LSEs [T, n_splits, H] f32.
@@ -131,7 +146,7 @@ int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t t
   // (the opt-in fp8 kernel keeps two workgroups per CU; every further split adds a partial to publish and fold)
   const bool few_fp8 = kv_format == SMLA_KV_FP8_B128 && n_heads <= 32 && few_fp8_enabled();
   const int slots = few_fp8 ? 2 * device_cus() : device_cus();
-  const bool wide = n_heads > 32 && ((kv_format == SMLA_KV_BF16 && wide_mode() != 0) || (kv_format == SMLA_KV_FP8_B128 && wide_mode() == 2));
+  const bool wide = n_heads > 32 && head_groups_enabled();
   const int per_wg = n_heads <= 32 ? 16 : (wide ? 128 : 64);
   const long long groups = (long long)n_tokens * ((n_heads + per_wg - 1) / per_wg);
   int want = (int)((slots + groups - 1) / groups);
@@ -150,12 +165,13 @@ static int fill_params(Params& p, const void* q, const void* kv, const int32_t* 
                        int32_t bt_stride, int64_t kv_seq_stride, int64_t kv_rows, float sm_scale) {
   p.q = q; p.kv = kv; p.indices = indices; p.seq_lens = nullptr; p.block_table = block_table; p.out = out; p.lse = lse;
   p.part_out = nullptr; p.part_lse = nullptr; p.counters = nullptr;
-  p.ws_header = static_cast<uint32_t*>(const_cast<void*>(q));   // (read, never used, when nothing is split)
+  p.ws_header = nullptr;                                        // (only a split launch has a workspace, and only it reads the header)
   p.n_tokens = n_tokens; p.tokens_per_seq = tokens_per_seq; p.n_heads = n_heads; p.topk = topk;
   p.page_size = block_table ? page_size : 1; p.bt_stride = block_table ? bt_stride : 0;
   p.n_splits = 1; p.split_len = topk;
   p.kv_seq_stride = kv_seq_stride; p.kv_rows = kv_rows; p.sm_scale = sm_scale; p.logit_cap = 0.f;
   p.token_band = token_bands_enabled() ? (n_tokens + 7) / 8 : 0;
+  p.merge_in_launch = 0;
   return SMLA_OK;
 }
 
@@ -202,12 +218,14 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
     p.ws_header = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(workspace) + SMLA_WS_HEADER_OFFSET);
     p.part_out = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + SMLA_WS_COUNTER_BYTES);
     p.part_lse = p.part_out + (size_t)n_tokens * n_splits * n_heads * d_v;
+    p.merge_in_launch = merge_in_launch_ok() ? 1 : 0;
   }
-  if (n_heads > 32 && wide_mode() == 2 && (kv_format == SMLA_KV_BF16 || kv_format == SMLA_KV_FP8_B128)) return launch_fwd_group(kv_format, p, s);
-  if (n_heads > 32 && wide_mode() == 1 && kv_format == SMLA_KV_BF16) return launch_fwd_wide(p, s);
-  if (n_heads > 32) return launch_fwd_tall(kv_format, p, s);
-  if (kv_format == SMLA_KV_FP8_B128 && few_fp8_enabled()) return launch_fwd_few_fp8(p, s);
-  return launch_fwd_short(kv_format, p, s);
+  if (n_heads > 32 && head_groups_enabled()) rc = launch_fwd_group(kv_format, p, s);
+  else if (n_heads > 32) rc = launch_fwd_tall(kv_format, p, s);
+  else if (kv_format == SMLA_KV_FP8_B128 && few_fp8_enabled()) rc = launch_fwd_few_fp8(p, s);
+  else rc = launch_fwd_short(kv_format, p, s);
+  if (rc != SMLA_OK || n_splits == 1 || p.merge_in_launch) return rc;
+  return launch_merge(p.part_out, p.part_lse, out, lse, n_tokens, n_heads, d_v, n_splits, s);
 }
 
 int smla_fwd(int kv_format, const void* q, const void* kv, const int32_t* indices,
@@ -273,7 +291,7 @@ int smla_merge_splits(const float* part_out, const float* part_lse, void* out, f
                       int32_t n_tokens, int32_t n_heads, int32_t d_v, int32_t n_splits,
                       void* stream) {
   if (!part_out || !part_lse || !out || !lse) return SMLA_EINVAL_NULLPTR;
-  if (n_tokens <= 0 || n_heads <= 0 || d_v != kDv || n_tokens > 65535) return SMLA_EINVAL_SHAPE;
+  if (n_tokens <= 0 || n_heads <= 0 || d_v != kDv || (long long)n_tokens * n_heads > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
   if (n_splits < 1 || n_splits > SMLA_MAX_SPLITS) return SMLA_EINVAL_SPLITS;
   if (!aligned16(part_out) || !aligned16(out)) return SMLA_EINVAL_ALIGN;
   return launch_merge(part_out, part_lse, out, lse, n_tokens, n_heads, d_v, n_splits,

@@ -28,13 +28,15 @@ struct Params {
   float* part_out;   // [T, n_splits, H, d_v] when n_splits > 1
   float* part_lse;   // [T, n_splits, H]
   unsigned long long* counters; // [T, ceil(H/64)] arrival tickets + published bits, zero between calls
-  uint32_t* ws_header;          // workspace header {magic, status, spin limit, -}; any readable word when n_splits == 1
+  uint32_t* ws_header;          // workspace header {magic, status, spin limit, -}; null (and never read) when n_splits == 1
   int32_t n_tokens, tokens_per_seq, n_heads, topk;
   int32_t page_size, bt_stride, n_splits, split_len;
   int64_t kv_seq_stride, kv_rows;
   float sm_scale;
   float logit_cap;              // > 0: every scaled score s becomes logit_cap * tanh(s / logit_cap) before the softmax
   int32_t token_band;           // 0: tokens dealt to the 8 XCDs in turn; > 0: XCD x takes tokens x*token_band .. (x+1)*token_band - 1
+  int32_t merge_in_launch;      // n_splits > 1 only.  1: the last split of a (token, head block) to arrive folds the others' partials
+                                // (needs all workgroups of a token behind one L2); 0: every split publishes, a second launch merges
 };
 
 // Which token a workgroup works on.  Block ids are dealt round-robin to the 8 XCDs (`xcd` = id % 8,
@@ -124,16 +126,30 @@ __device__ __forceinline__ void ws_flag(const Params& p, uint32_t bits) {
   __hip_atomic_fetch_or(p.ws_header + 1, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// One thread of the workgroup: take an arrival ticket and decide the workgroup's role.  `magic`
-// is the header's first word as read at kernel entry.  An inconsistent word (more arrivals than
-// splits, my own bit or a bit past the last split already set, more published than arrived)
-// flags the workspace and zeroes the word (the host re-initialises a flagged workspace: a split
-// that arrives after this may leave its ticket behind).
-__device__ __forceinline__ int ws_arrive(const Params& p, unsigned long long* word, uint32_t magic, int ns, int sp) {
-  if (magic != kWsMagic) {
+// The header's magic and status words as they stood when the kernel started (one 8-byte load, long
+// before the split merge needs it).  A launch that does not split has no workspace and reads nothing.
+struct WsHead { uint32_t magic, status; };
+__device__ __forceinline__ WsHead ws_read_head(const Params& p) {
+  if (p.n_splits <= 1 || !p.merge_in_launch) return WsHead{0u, 0u};
+  const uint2 h = *reinterpret_cast<const uint2*>(p.ws_header);
+  return WsHead{h.x, h.y};
+}
+
+// One thread of the workgroup: take an arrival ticket and decide the workgroup's role.  `head`
+// is the header as read at kernel entry.  A workspace that an earlier launch has flagged stays
+// unusable until the host has looked at it (smla_workspace_status re-initialises it): a launch
+// that gave up may have left tickets or published bits behind, and a word in such a state can
+// look legal to the next launch, which would then fold in a stale partial.  So a non-zero status
+// makes every split of every later launch give up at once, without touching the word.
+// An inconsistent word (more arrivals than splits, my own bit or a bit past the last split already
+// set, more published than arrived) flags the workspace and zeroes the word.
+__device__ __forceinline__ int ws_arrive(const Params& p, unsigned long long* word, WsHead head, int ns, int sp) {
+  if (!p.merge_in_launch) return kRolePublish;       // a second launch merges: nothing to agree on
+  if (head.magic != kWsMagic) {
     ws_flag(p, SMLA_WS_STATUS_UNINITIALISED);
     return kRoleError;
   }
+  if (head.status != 0) return kRoleError;
   const unsigned long long old = __hip_atomic_fetch_add(word, 1ull << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const uint32_t ticket = (uint32_t)(old >> 32), bits = (uint32_t)old;
   const uint32_t legal = ns >= 32 ? 0xffffffffu : (1u << ns) - 1u;
@@ -143,6 +159,11 @@ __device__ __forceinline__ int ws_arrive(const Params& p, unsigned long long* wo
     return kRoleError;
   }
   return ticket == (uint32_t)ns - 1 ? kRoleLast : kRolePublish;
+}
+
+// One thread of a publishing workgroup, after its partial's stores have been acknowledged.
+__device__ __forceinline__ void ws_publish(const Params& p, unsigned long long* word, int sp) {
+  if (p.merge_in_launch) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // One thread of the last workgroup to arrive: poll until every other split has published, at
@@ -211,7 +232,6 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
 int launch_fwd_scalar(int kv_format, const Params& p, hipStream_t s);
 int launch_fwd_tall(int kv_format, const Params& p, hipStream_t s);    // n_heads > 32 (logit cap: a second instantiation)
 int launch_fwd_short(int kv_format, const Params& p, hipStream_t s);   // n_heads <= 32
-int launch_fwd_wide(const Params& p, hipStream_t s);                   // n_heads > 32, bf16 rows, 128 heads per workgroup, 8 wavefronts (opt-in)
 int launch_fwd_group(int kv_format, const Params& p, hipStream_t s);   // n_heads > 32, bf16 rows or fp8 records, 128 heads per workgroup, a wavefront per 32 heads (opt-in)
 int launch_fwd_few_fp8(const Params& p, hipStream_t s);                // n_heads <= 32, fp8 records, two workgroups per CU (opt-in)
 int launch_merge(const float* part_out, const float* part_lse, void* out, float* lse,

@@ -127,7 +127,7 @@ __global__ __launch_bounds__(kNT, 2) void fwd_few_fp8_kernel(Params p, int n_hbl
   const int head = head0 + l16;
   const bool head_ok = head < p.n_heads;
   const uint8_t* kv = static_cast<const uint8_t*>(p.kv);
-  const uint32_t ws_magic = *p.ws_header;    // read long before the split merge needs it
+  const WsHead ws_head = ws_read_head(p);    // read long before the split merge needs it
   const bool scorer = wave < 2;              // wavefronts 0, 1: tokens 16 wave .. + 15 of every tile
 
   // ---- the first chunk's index loads go out before anything else
@@ -381,11 +381,15 @@ __global__ __launch_bounds__(kNT, 2) void fwd_few_fp8_kernel(Params p, int n_hbl
   // ---- split merge inside the launch (protocol and failure handling: ws_arrive / ws_wait_published)
   const int ns = p.n_splits;
   unsigned long long* word = p.counters + (size_t)t * n_hblocks + hb;
-  if (tid == 0) s_nvalid = ws_arrive(p, word, ws_magic, ns, sp);
+  if (tid == 0) s_nvalid = ws_arrive(p, word, ws_head, ns, sp);
   __syncthreads();
   const int role = s_nvalid;
-  auto give_up = [&]() {
+  auto give_up = [&]() {                     // the workspace was not what it should be: mark the rows (NaN LSE, zero output)
     if (wave == 0 && q4 == 0 && head_ok) p.lse[(size_t)t * p.n_heads + head] = __uint_as_float(0x7fc00000u);
+    if (row_ok) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) store_final(j, make_float4(0.f, 0.f, 0.f, 0.f));
+    }
   };
   if (role == kRoleError) { give_up(); return; }
   if (role == kRolePublish) {
@@ -402,7 +406,7 @@ __global__ __launch_bounds__(kNT, 2) void fwd_few_fp8_kernel(Params p, int n_hbl
     }
     hw::wait_vmcnt<0>();
     __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) ws_publish(p, word, sp);
     return;
   }
   if (tid == 0) s_flag = ws_wait_published(p, word, ns, sp) ? 0 : 1;

@@ -241,7 +241,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   const int head0 = hb * 128 + wave * 32;                         // first head of this wavefront
   const uint8_t* kv = static_cast<const uint8_t*>(p.kv);
   const int k_begin = sp * p.split_len, k_end = min(k_begin + p.split_len, p.topk);
-  const uint32_t ws_magic = *p.ws_header;    // read long before the split merge needs it
+  const WsHead ws_head = ws_read_head(p);    // read long before the split merge needs it
 
   // ---- the first chunk's index loads go out before anything else: the row list they lead to
   // (index -> page table -> row fetch) is the longest dependent chain of the kernel
@@ -585,7 +585,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   // = row), read back one head row at a time, 8 consecutive columns per lane.
   __syncthreads();                           // the ring is free
   if (p.n_splits > 1 && tid == 0)
-    s_nvalid = ws_arrive(p, p.counters + (size_t)t * n_hblocks + hb, ws_magic, p.n_splits, sp);
+    s_nvalid = ws_arrive(p, p.counters + (size_t)t * n_hblocks + hb, ws_head, p.n_splits, sp);
   const int lane_e = hw::lane_id();          // (lane coordinates retaken here rather than carried through the loop)
   const int l16_e = lane_e & 15, q4_e = lane_e >> 4;
   float lse_nat[2];                          // of heads 16 ht + l16
@@ -647,10 +647,12 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   unsigned long long* word = p.counters + (size_t)t * n_hblocks + hb;
   __syncthreads();                                                 // the ticket lane 0 of wavefront 0 took at the top of the epilogue is in s_nvalid
   const int role = s_nvalid;
-  auto give_up = [&]() {
+  auto give_up = [&]() {                                           // mark the rows: NaN LSE, zero output
 #pragma unroll
     for (int ht = 0; ht < 2; ++ht)
       if (q4_e == 0 && head_ok(ht)) p.lse[lse_index(ht)] = __uint_as_float(0x7fc00000u);
+    const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int row = 0; row < n_rows; ++row) store_bf16x8(row, z, z);
   };
   if (role == kRoleError) { give_up(); return; }
   if (role == kRolePublish) {
@@ -670,7 +672,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
     }
     hw::wait_vmcnt<0>();
     __syncthreads();
-    if (wave == 0 && lane_e == 0) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wave == 0 && lane_e == 0) ws_publish(p, word, sp);
     return;
   }
   // last arrival: wait for the others, then fold the normalised partials in split order with every

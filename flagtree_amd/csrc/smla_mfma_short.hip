@@ -175,7 +175,7 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
   const int head = head0 + l16;
   const bool head_ok = head < p.n_heads;
   const uint8_t* kv = static_cast<const uint8_t*>(p.kv);
-  const uint32_t ws_magic = *p.ws_header;    // read long before the split merge needs it
+  const WsHead ws_head = ws_read_head(p);    // read long before the split merge needs it
 
   // ---- the first chunk's index loads go out before anything else: the row list they lead to
   // (index -> page table -> row fetch) is the longest dependent chain of the kernel
@@ -472,11 +472,15 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
   // rows' LSE with NaN, see ws_arrive / ws_wait_published).
   const int ns = p.n_splits;
   unsigned long long* word = p.counters + (size_t)t * n_hblocks + hb;
-  if (tid == 0) s_nvalid = ws_arrive(p, word, ws_magic, ns, sp);
+  if (tid == 0) s_nvalid = ws_arrive(p, word, ws_head, ns, sp);
   __syncthreads();
   const int role = s_nvalid;
-  auto give_up = [&]() {                     // the workspace was not what it should be: mark the rows
+  auto give_up = [&]() {                     // the workspace was not what it should be: mark the rows (NaN LSE, zero output)
     if (wave == 0 && q4 == 0 && head_ok) p.lse[(size_t)t * p.n_heads + head] = __uint_as_float(0x7fc00000u);
+    if (row_ok) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) store_final(j, make_float4(0.f, 0.f, 0.f, 0.f));
+    }
   };
   if (role == kRoleError) { give_up(); return; }
   if (role == kRolePublish) {
@@ -494,7 +498,7 @@ __global__ __launch_bounds__(kNT) void fwd_short_kernel(Params p, int n_hblocks)
     }
     hw::wait_vmcnt<0>();
     __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) ws_publish(p, word, sp);
     return;
   }
   // last arrival: every other split holds a ticket, so it is running and will publish.  Wait for

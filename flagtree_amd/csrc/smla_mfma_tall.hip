@@ -285,7 +285,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   const bool head_ok = head < p.n_heads;
   const uint8_t* kv = static_cast<const uint8_t*>(p.kv);
   const int k_begin = sp * p.split_len, k_end = min(k_begin + p.split_len, p.topk);
-  const uint32_t ws_magic = *p.ws_header;    // read long before the split merge needs it
+  const WsHead ws_head = ws_read_head(p);    // read long before the split merge needs it
 
   // ---- the first chunk's index loads go out before anything else: the row list they lead to
   // (index -> page table -> row fetch) is the longest dependent chain of the kernel
@@ -667,7 +667,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // the arrival ticket of the split merge is taken here, so that its round trip to memory
   // overlaps the staging below (the merge itself is described further down)
   if (p.n_splits > 1 && tid_e == 0)
-    s_nvalid = ws_arrive(p, p.counters + (size_t)t * n_hblocks + hb, ws_magic, p.n_splits, sp);
+    s_nvalid = ws_arrive(p, p.counters + (size_t)t * n_hblocks + hb, ws_head, p.n_splits, sp);
 #pragma unroll
   for (int ht = 0; ht < 2; ++ht) {
     float l = l_part[ht];
@@ -726,8 +726,9 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   const int ns = p.n_splits;
   unsigned long long* word = p.counters + (size_t)t * n_hblocks + hb;
   const int role = s_nvalid;                                       // ticket taken at the top of the epilogue
-  auto give_up = [&]() {                                           // the workspace was not what it should be: mark the rows
+  auto give_up = [&]() {                                           // the workspace was not what it should be: mark the rows (NaN LSE, zero output)
     if (dh == 0 && g_e == 0 && head_ok_e) p.lse[(size_t)t * p.n_heads + head_e] = __uint_as_float(0x7fc00000u);
+    for (int row = 0; row < n_rows; ++row) store_bf16x4(row, make_float4(0.f, 0.f, 0.f, 0.f));
   };
   if (role == kRoleError) { give_up(); return; }
   if (role == kRolePublish) {
@@ -743,7 +744,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     }
     hw::wait_vmcnt<0>();
     __syncthreads();
-    if (tid_e == 0) __hip_atomic_fetch_or(word, 1ull << sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid_e == 0) ws_publish(p, word, sp);
     return;
   }
   // last arrival: every other split holds a ticket, so it is running and will publish.  Wait for

@@ -178,7 +178,7 @@ __global__ __launch_bounds__(128) void merge_kernel(const float* __restrict__ pa
                                                     const float* __restrict__ part_lse,
                                                     uint16_t* __restrict__ out, float* __restrict__ lse,
                                                     int n_heads, int n_splits) {
-  const int h = blockIdx.x, t = blockIdx.y;
+  const int h = blockIdx.x % n_heads, t = blockIdx.x / n_heads;
   float m = -INFINITY;
   for (int i = 0; i < n_splits; ++i)
     m = fmaxf(m, part_lse[((size_t)t * n_splits + i) * n_heads + h]);
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(128) void merge_kernel(const float* __restrict__ pa
 int launch_merge(const float* part_out, const float* part_lse, void* out, float* lse, int n_tokens,
                  int n_heads, int d_v, int n_splits, hipStream_t s) {
   if (d_v != kDv) return SMLA_EINVAL_SHAPE;
-  dim3 grid(n_heads, n_tokens), block(128);
+  dim3 grid((unsigned)n_heads * (unsigned)n_tokens), block(128);
   hipLaunchKernelGGL(merge_kernel, grid, block, 0, s, part_out, part_lse, static_cast<uint16_t*>(out), lse, n_heads,
                                       n_splits);
   return hip_status(hipGetLastError());

@@ -122,10 +122,23 @@ def make_workspace(n_bytes, device):
     return ws
 
 
-def workspace_status(workspace):
+def workspace_status(workspace=None, device=None):
     """Wait for the current stream and report what the split launches left in ``workspace``'s header.
     Returns 0 when healthy; otherwise raises RuntimeError naming the SMLA_WS_STATUS bits, after the
-    library has initialised the workspace again."""
+    library has initialised the workspace again.
+
+    ``workspace=None`` checks the workspace ``sparse_mla_fwd`` / ``decode_attention_fwd`` keep for
+    the current stream of ``device`` (default: the current device); 0 when no split launch has
+    needed one yet.  A launch whose merge gave up marks its rows with a NaN LSE and flags the
+    workspace, and every later split launch on that workspace gives up too until this function has
+    run: a serving loop calls it wherever it synchronises anyway (it waits for the stream)."""
+    if workspace is None:
+        device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        if device.type == "cuda" and device.index is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        workspace = _workspaces.get((device, _lib.stream_handle(device)))
+        if workspace is None:
+            return 0
     _check_workspace(workspace, 0, workspace.device)
     import ctypes
     status = ctypes.c_uint32(0)

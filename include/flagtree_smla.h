@@ -93,7 +93,8 @@ int smla_abi_version(void);
  *               smla_workspace_bytes() bytes (device, 16-byte aligned) that went through
  *               smla_workspace_init() once; the split results are merged inside the same launch
  *               by the last workgroup to finish, which also leaves the workspace ready for the
- *               next call.  Calls that share a workspace must not overlap.
+ *               next call (or by a second launch on the same stream: smla_merge_in_launch).
+ *               Calls that share a workspace must not overlap.
  *   sm_scale    positive and finite.
  * Stands where the reference's host wrapper launches its attention kernel
  * (/root/reference/python/triton/ops/flash_attention.py:387-408; MLA decode:
@@ -137,6 +138,20 @@ int smla_fwd_scalar(int kv_format, const void* q, const void* kv, const int32_t*
 /* Split count smla_fwd picks for n_splits = 0 on the current device. */
 int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t topk);
 
+/*
+ * How a split launch is merged on the current device: 1 = inside the launch, 0 = by a second
+ * launch (the smla_merge_splits kernel) right behind it on the same stream.
+ * The merge inside the launch hands partials from workgroup to workgroup through the L2 cache
+ * without fences, so it needs every workgroup of a token behind one L2.  Assumption it rests on:
+ * block ids are dealt round-robin to the device's XCDs, the kernels give a token's workgroups ids
+ * 8 apart, and the XCD count divides 8.  That holds for a gfx950 device of 256, 128, 64 or at most
+ * 32 compute units (a whole MI355X or one of its partitions); on any other compute-unit count, or
+ * with FLAGTREE_SMLA_SEPARATE_MERGE=1 in the environment, the second launch is used.
+ * No counterpart in the reference, whose stage 2 is always a second launch
+ * (test_accuracy_musa_vllm_mla.py:426-477).
+ */
+int smla_merge_in_launch(void);
+
 /* Bytes of workspace smla_fwd needs for the given split count (0 when n_splits <= 1). */
 size_t smla_workspace_bytes(int32_t n_tokens, int32_t n_heads, int32_t d_v, int32_t n_splits);
 
@@ -150,12 +165,14 @@ int smla_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
  * workspace without its magic word, an arrival word in an illegal state, or whose last split
  * waits longer than the header's poll limit for the others does not hang and does not merge: it
  * sets a SMLA_WS_STATUS_* bit in the header, writes NaN to the LSE of the rows concerned and
- * ends normally; until the host has dealt with it, later launches on that workspace may be
- * flagged too.  This call waits for `stream`, copies the header back, stores the status bits in
+ * ends normally.  A flagged workspace stays unusable until the host has dealt with it: every
+ * later split launch on it gives up at once (NaN LSE, `out` rows zero or untouched), because a
+ * launch that gave up may have left arrival words in a state the next one cannot tell from a
+ * legal one.  This call waits for `stream`, copies the header back, stores the status bits in
  * *status_out (may be NULL) and returns SMLA_OK when they were zero; otherwise it initialises
  * the workspace again (as smla_workspace_init does, unless the magic word was missing) and
- * returns SMLA_EWORKSPACE_STATE.  It synchronises, so it is for tests, set-up code and error
- * handling, not for the serving loop.
+ * returns SMLA_EWORKSPACE_STATE.  It synchronises, so a serving loop calls it at the points where
+ * it synchronises anyway (after a batch has been read back), or when it meets a NaN LSE.
  * No counterpart in the reference (its two-stage decode keeps no state between launches:
  * test_accuracy_musa_vllm_mla.py:426-477 is a second launch).
  */

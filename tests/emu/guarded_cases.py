@@ -29,7 +29,7 @@ def _guard_cfg(cfg, end):
 
 def forward_case(make, n_splits, dense=False, env=None):
     def run(end):
-        for k in ("FLAGTREE_SMLA_FEW_FP8", "FLAGTREE_SMLA_WIDE"):
+        for k in ("FLAGTREE_SMLA_FEW_FP8", "FLAGTREE_SMLA_HEAD_GROUPS"):
             os.environ.pop(k, None)
         os.environ.update(env or {})
         cfg = make()
@@ -134,20 +134,16 @@ CASES = {
     # 65 heads: the second head group of the second block lies wholly past the last head
     "tall_bf16_empty_head_group_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=65, pages_per_seq=5, topk=200, pad_frac=0.06), 3),
     "tall_fp8_split": forward_case(lambda: fp8_cfg(2, 128, 4, 150), 2),
-    "group_fp8_split": forward_case(lambda: fp8_cfg(2, 128, 4, 150), 2, env={"FLAGTREE_SMLA_WIDE": "2"}),
-    "group_fp8_short_lists": forward_case(lambda: fp8_cfg(3, 65, 2, 40), 1, env={"FLAGTREE_SMLA_WIDE": "2"}),
+    "group_fp8_split": forward_case(lambda: fp8_cfg(2, 128, 4, 150), 2, env={"FLAGTREE_SMLA_HEAD_GROUPS": "1"}),
+    "group_fp8_short_lists": forward_case(lambda: fp8_cfg(3, 65, 2, 40), 1, env={"FLAGTREE_SMLA_HEAD_GROUPS": "1"}),
     "tall_fp8_short_lists": forward_case(lambda: fp8_cfg(3, 65, 2, 40), 1),
     "short_bf16_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=2, heads=16, pages_per_seq=5, topk=200, pad_frac=0.06), 2),
     "short_bf16_ragged_heads": forward_case(lambda: workloads.decode_bf16("cpu", batch=1, heads=9, pages_per_seq=5, topk=150, pad_frac=0.06), 1),
     "short_fp8_split": forward_case(lambda: fp8_cfg(2, 16, 4, 150), 2),
-    "wide_bf16_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=2, heads=128, pages_per_seq=5, topk=200, pad_frac=0.06), 2,
-                                    env={"FLAGTREE_SMLA_WIDE": "1"}),
     "group_bf16_split": forward_case(lambda: workloads.decode_bf16("cpu", batch=2, heads=128, pages_per_seq=5, topk=200, pad_frac=0.06), 2,
-                                      env={"FLAGTREE_SMLA_WIDE": "2"}),
+                                      env={"FLAGTREE_SMLA_HEAD_GROUPS": "1"}),
     "group_bf16_ragged": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=65, pages_per_seq=5, topk=90, pad_frac=0.06), 3,
-                                       env={"FLAGTREE_SMLA_WIDE": "2"}),
-    "wide_bf16_ragged": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=65, pages_per_seq=5, topk=90, pad_frac=0.06), 3,
-                                     env={"FLAGTREE_SMLA_WIDE": "1"}),
+                                       env={"FLAGTREE_SMLA_HEAD_GROUPS": "1"}),
     "few_fp8_split": forward_case(lambda: fp8_cfg(2, 16, 4, 150), 2, env={"FLAGTREE_SMLA_FEW_FP8": "1"}),
     "few_fp8_ragged_heads": forward_case(lambda: fp8_cfg(1, 9, 4, 100), 1, env={"FLAGTREE_SMLA_FEW_FP8": "1"}),
     "dense_tall": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=128, pages_per_seq=3, topk=64), 2, dense=True),

@@ -145,11 +145,11 @@ def test_many_heads_fp8_pipeline_at_every_tile_count(topk, n_splits):
                                                  (200, 3, 128), (1030, 1, 40), (2100, 2, 128)])
 def test_head_group_kernel_fp8_pipeline(topk, n_splits, heads, monkeypatch):
     """The same raw-record pipeline inside the wavefront-per-head-group kernel (its own row xor)."""
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "2")
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")
     cfg, _ = _fp8_cfg(1, heads, 40, topk, pad_frac=0.0 if topk < 40 else 0.04)
     out, lse = _forward_all_ways(cfg, n_splits)
     _check(cfg, out, lse)
-    os.environ.pop("FLAGTREE_SMLA_WIDE")
+    os.environ.pop("FLAGTREE_SMLA_HEAD_GROUPS")
     out1, lse1, rc = harness.forward(cfg, n_splits=n_splits)             # the first kernel
     assert rc == 0 and max_abs(to_np(out1), to_np(out)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse)) <= 1e-5
 
@@ -157,7 +157,7 @@ def test_head_group_kernel_fp8_pipeline(topk, n_splits, heads, monkeypatch):
 @pytest.mark.parametrize("mode", ["first", "wavefront_per_head_group"])
 def test_many_heads_fp8_redo_passes(mode, monkeypatch):
     if mode != "first":
-        monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "2")
+        monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")
     _many_heads_fp8_redo_passes()
 
 
@@ -184,11 +184,10 @@ def _many_heads_fp8_redo_passes():
         assert max_abs(to_np(out).reshape(ro.shape), ro) <= 1.2e-2 * max(1.0, float(np.abs(ro).max()))
 
 
-@pytest.fixture(params=["1", "2"], ids=["eight_wavefronts", "wavefront_per_head_group"])
-def wide_kernel(request, monkeypatch):
-    """Routes many-heads bf16 launches to one of the two 128-heads-per-workgroup kernels (opt-in
-    until they are measured)."""
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", request.param)
+@pytest.fixture
+def wide_kernel(monkeypatch):
+    """Routes many-heads launches to the 128-heads-per-workgroup kernel (opt-in until it is measured)."""
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")
 
 
 @pytest.mark.parametrize("heads,n_splits,topk", [(128, 1, 300), (128, 2, 300), (64, 3, 200), (96, 1, 100), (40, 2, 70),
@@ -198,7 +197,7 @@ def test_128_heads_per_workgroup_kernel(wide_kernel, heads, n_splits, topk):
     cfg = workloads.decode_bf16("cpu", batch=2, heads=heads, pages_per_seq=20, topk=topk, pad_frac=0.07)
     out, lse = _forward_all_ways(cfg, n_splits)
     _check(cfg, out, lse)
-    os.environ.pop("FLAGTREE_SMLA_WIDE")
+    os.environ.pop("FLAGTREE_SMLA_HEAD_GROUPS")
     out1, lse1, rc = harness.forward(cfg, n_splits=n_splits)             # the first kernel: same results to the bar, not to the bit
     # (it sums in another order, so somewhere a last bit differs: the switch did select another kernel)
     assert rc == 0 and not (torch.equal(out1.view(torch.int16), out.view(torch.int16)) and torch.equal(lse1, lse))
@@ -347,7 +346,7 @@ def test_causal_prefill_reduced():
     _check(cfg, out, lse)
 
 
-@pytest.mark.parametrize("wide", ["0", "1", "2"])
+@pytest.mark.parametrize("wide", ["0", "1"])
 @pytest.mark.parametrize("heads,n_splits", [(128, 1), (128, 2), (16, 1), (16, 3)])
 def test_token_bands_only_change_which_workgroup_takes_a_token(heads, n_splits, wide, monkeypatch):
     """FLAGTREE_SMLA_TOKEN_BANDS=1 hands each XCD a contiguous band of tokens instead of every
@@ -355,8 +354,8 @@ def test_token_bands_only_change_which_workgroup_takes_a_token(heads, n_splits, 
     bits (43 tokens: bands of 6, the last one short, some workgroups without a token)."""
     from flagtree_amd import workloads
     if heads == 16 and wide != "0":
-        pytest.skip("the 128-heads kernels do not take 16 heads")
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", wide)
+        pytest.skip("the 128-heads kernel does not take 16 heads")
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", wide)
     cfg = workloads.prefill_causal_bf16("cpu", tokens=43, heads=heads, topk=300 if n_splits > 1 else 48)
     out0, lse0, rc = harness.forward(cfg, n_splits=n_splits)
     assert rc == 0
@@ -458,7 +457,7 @@ def test_dense_decode_with_logit_cap(heads, fmt, std, cap, min_diff):
 
 
 @pytest.mark.parametrize("seed", list(range(12)))
-@pytest.mark.parametrize("few_fp8", [False, True, "wide", "wide_k"])
+@pytest.mark.parametrize("few_fp8", [False, True, "head_groups"])
 def test_random_shapes_against_oracle(seed, few_fp8, monkeypatch):
     """Seeded draws over head counts, list lengths, page sizes, tokens per sequence, split counts,
     padding patterns, page tables with holes and both cache formats (the GPU suite's recipe at sizes
@@ -474,10 +473,10 @@ def test_random_shapes_against_oracle(seed, few_fp8, monkeypatch):
     n_splits = [1, 2, 3, 5][int(rng.integers(4))]
     paged = rng.random() < 0.7
     ctx = int(rng.choice([64, 300, 1200]))
-    if few_fp8 in ("wide", "wide_k"):
-        if heads <= 32 or (fmt != "bf16" and few_fp8 == "wide"):
-            pytest.skip("the opt-in kernels cover many heads (the eight-wavefront one over a bf16 cache only)")
-        monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1" if few_fp8 == "wide" else "2")
+    if few_fp8 == "head_groups":
+        if heads <= 32:
+            pytest.skip("the opt-in kernel covers many heads")
+        monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")
     elif few_fp8:
         if fmt != "fp8_e4m3_b128" or heads > 32:
             pytest.skip("the opt-in kernel covers few heads over an fp8 cache")
@@ -547,15 +546,15 @@ def _header(ws):
     return ws[_lib.SMLA_WS_HEADER_OFFSET:_lib.SMLA_WS_HEADER_OFFSET + 16].view(torch.int32)
 
 
-@pytest.mark.parametrize("kernel", ["many_heads", "eight_wavefronts", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split"])
+@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split"])
 def test_merging_workgroup_really_waits_for_the_others(kernel, monkeypatch):
     """With one workgroup at a time the last arrival of a split merge always finds the others'
     partials published.  Here several share the machine and are switched every few steps: the
     merging workgroup polls, the others publish meanwhile (the poll count says it happened), and
     the results are the same bits as without any waiting."""
     from flagtree_amd import workloads
-    heads = 128 if kernel in ("many_heads", "eight_wavefronts", "wavefront_per_head_group") else 16
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", {"eight_wavefronts": "1", "wavefront_per_head_group": "2"}.get(kernel, "0"))
+    heads = 128 if kernel in ("many_heads", "wavefront_per_head_group") else 16
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel == "wavefront_per_head_group" else "0")
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel == "few_heads_fp8_column_split" else "0")
     if kernel == "few_heads_fp8_column_split":
         cfg, _ = _fp8_cfg(3, heads, 20, 400, pad_frac=0.05)
@@ -598,12 +597,96 @@ def test_stale_arrival_word_is_flagged_not_hung(heads, stale, schedule):
     per_block = 64 if heads > 32 else 16
     l = to_np(lse)
     assert np.isnan(l[1, :min(per_block, heads)]).all()
-    assert max_abs(l[[0, 2]], to_np(ref_lse)[[0, 2]]) <= 1e-3
+    # workgroups that started after the flag went up give up as well (here they run one after the
+    # other, on the GPU most start together): every other row is either right or marked, never wrong
+    others = l[[0, 2]]
+    assert (np.isnan(others) | (np.abs(others - to_np(ref_lse)[[0, 2]]) <= 1e-3)).all()
+    marked = np.isnan(l)
+    assert not to_np(out).reshape(3, heads, 512)[marked].any()           # marked rows are zero
     assert harness.workspace_status(ws) == (0, 0)
     assert int((_words(ws) != 0).sum()) == 0
     out2, lse2, rc = harness.forward(cfg, n_splits=2, workspace=ws)
     assert rc == 0 and harness.workspace_status(ws) == (0, 0)
     assert max_abs(to_np(lse2), to_np(ref_lse)) <= 1e-3 and max_abs(to_np(out2), to_np(ref_out)) <= 1e-2
+
+
+@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split"])
+def test_flagged_workspace_stays_loud_until_the_host_has_looked(kernel, monkeypatch):
+    """A launch that gave up may leave an arrival word in a state the next launch cannot tell from
+    a legal one: here one ticket and the OTHER split's published bit, with two splits.  Judged by
+    the word alone, this split would draw the last ticket, find the bit set and fold in whatever
+    the partial buffer holds.  The status word the first launch left makes every split give up
+    instead (NaN LSE, zero output) until smla_workspace_status has run."""
+    from flagtree_amd import _lib, workloads
+    heads = 128 if kernel in ("many_heads", "wavefront_per_head_group") else 16
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel == "wavefront_per_head_group" else "0")
+    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel == "few_heads_fp8_column_split" else "0")
+    if kernel == "few_heads_fp8_column_split":
+        cfg, _ = _fp8_cfg(2, heads, 6, 260, pad_frac=0.05)
+    else:
+        cfg = workloads.decode_bf16("cpu", batch=2, heads=heads, pages_per_seq=6, topk=260, pad_frac=0.05)
+    ref_out, ref_lse, rc = harness.forward(cfg, n_splits=1)
+    assert rc == 0
+    ws = harness.make_workspace(harness.lib().smla_workspace_bytes(2, heads, 512, 2))
+    ws[_lib.SMLA_WS_COUNTER_BYTES:] = 0x3C                   # partials nobody wrote: finite garbage
+    _header(ws)[1] = 4                                        # what a timed-out merge leaves
+    _words(ws)[:] = (1 << 32) | 2                             # ... and a late publisher of split 1
+    out, lse, rc = harness.forward(cfg, n_splits=2, workspace=ws)
+    assert rc == 0
+    assert np.isnan(to_np(lse)).all() and not to_np(out).any()
+    assert int((_words(ws) != ((1 << 32) | 2)).sum()) == 0    # nobody took a ticket
+    rc, status = harness.workspace_status(ws)
+    assert rc == _lib.SMLA_EWORKSPACE_STATE and status == 4
+    assert harness.workspace_status(ws) == (0, 0) and int((_words(ws) != 0).sum()) == 0
+    out2, lse2, rc = harness.forward(cfg, n_splits=2, workspace=ws)
+    assert rc == 0 and harness.workspace_status(ws) == (0, 0)
+    assert max_abs(to_np(lse2), to_np(ref_lse)) <= 1e-3 and max_abs(to_np(out2), to_np(ref_out)) <= 1e-2
+
+
+@pytest.mark.parametrize("how", ["compute units of an unknown layout", "environment"])
+@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split"])
+def test_splits_merged_by_a_second_launch(kernel, how, monkeypatch, schedule):
+    """The merge inside the launch needs all workgroups of a token behind one L2, which the library
+    only claims for compute-unit counts it knows the XCD layout of.  Elsewhere (here: 48 compute
+    units), or when asked to, every split publishes and the merge kernel runs as a second launch:
+    same results to the bar, arrival words never touched, and an uninitialised workspace is fine."""
+    from flagtree_amd import workloads
+    heads = 128 if kernel in ("many_heads", "wavefront_per_head_group") else 16
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel == "wavefront_per_head_group" else "0")
+    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel == "few_heads_fp8_column_split" else "0")
+    if kernel == "few_heads_fp8_column_split":
+        cfg, _ = _fp8_cfg(3, heads, 6, 330, pad_frac=0.05)
+    else:
+        cfg = workloads.decode_bf16("cpu", batch=3, heads=heads, pages_per_seq=6, topk=330, pad_frac=0.05)
+    lib = harness.lib()
+    assert lib.smla_merge_in_launch() == 1
+    out1, lse1, rc = harness.forward(cfg, n_splits=3)
+    assert rc == 0
+    try:
+        if how == "environment":
+            monkeypatch.setenv("FLAGTREE_SMLA_SEPARATE_MERGE", "1")
+        else:
+            lib.emu_set_cu_count(48)
+        assert lib.smla_merge_in_launch() == 0
+        ws = torch.full((lib.smla_workspace_bytes(3, heads, 512, 3),), 0x3C, dtype=torch.uint8)     # never initialised
+        launches = lib.emu_launch_count()
+        out, lse, rc = harness.forward(cfg, n_splits=3, workspace=ws)
+        assert rc == 0 and lib.emu_launch_count() - launches == 2
+        assert int((_words(ws) != 0x3C3C3C3C3C3C3C3C).sum()) == 0 and int((_header(ws) != 0x3C3C3C3C).sum()) == 0
+    finally:
+        lib.emu_set_cu_count(harness.EMU_CUS)
+    _check(cfg, out, lse)
+    assert max_abs(to_np(out), to_np(out1)) <= 2e-3 and max_abs(to_np(lse), to_np(lse1)) <= 1e-5
+
+
+def test_merge_inside_the_launch_only_on_known_compute_unit_counts():
+    lib = harness.lib()
+    try:
+        for n, want in ((16, 1), (32, 1), (64, 1), (128, 1), (256, 1), (20, 1), (48, 0), (96, 0), (240, 0), (304, 0)):
+            lib.emu_set_cu_count(n)
+            assert lib.smla_merge_in_launch() == want, n
+    finally:
+        lib.emu_set_cu_count(harness.EMU_CUS)
 
 
 def test_uninitialised_workspace_is_flagged(schedule):
@@ -710,6 +793,29 @@ def test_local_gemm(m, n, k, chunks):
     harness.configure()
 
 
+def test_local_gemm_on_a_compute_unit_count_that_is_no_multiple_of_eight():
+    """24 tiles on 20 compute units leave a rest of 4 tiles, few enough to be halved; but the half-tile
+    mapping needs the whole tiles to come in groups of 8, which 20 does not give: all tiles stay
+    whole, every one is computed once."""
+    m, n, k = 2048, 768, 128
+    g = torch.Generator().manual_seed(99)
+    x = (torch.randn((m, k), generator=g) * 0.1).to(torch.bfloat16)
+    w = (torch.randn((k, n), generator=g) * 0.1).to(torch.bfloat16)
+    partial = torch.randn((m, n), generator=g)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16)
+    lib = harness.lib()
+    try:
+        lib.emu_set_cu_count(20)
+        harness.work_counts()
+        rc = lib.smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), partial.data_ptr(), out.data_ptr(), m, n, k, 2, (m // 2) * n, None)
+        flops = harness.work_counts()["mfma_flops"]
+    finally:
+        lib.emu_set_cu_count(harness.EMU_CUS)
+    assert rc == 0 and flops == 2.0 * m * n * k               # nothing twice, nothing left out
+    want = oracle.gemm_rs_local(to_np(x), to_np(w), to_np(partial), n_chunks=2).reshape(m, n)
+    assert max_abs(to_np(out), want) <= 1e-2 + 1e-2 * float(np.abs(want).max())
+
+
 # ---- memory safety: every buffer between inaccessible pages ------------------------------------
 
 def test_no_entry_point_touches_memory_outside_its_buffers():
@@ -747,7 +853,7 @@ def _bank_ratio(stats):
     return {k: v[1] / v[2] for k, v in stats.items() if v[0]}
 
 
-@pytest.mark.parametrize("mode", ["first", "eight_wavefronts", "wavefront_per_head_group", "first_fp8", "wavefront_per_head_group_fp8"])
+@pytest.mark.parametrize("mode", ["first", "wavefront_per_head_group", "first_fp8", "wavefront_per_head_group_fp8"])
 def test_many_heads_kernels_address_lds_without_bank_conflicts(mode, monkeypatch):
     """The emulator prices every LDS access the kernels make by address (fragment reads, transposing
     reads, probability writes) the way the hardware serves it: 16-byte accesses 16 lanes at a time,
@@ -759,7 +865,7 @@ def test_many_heads_kernels_address_lds_without_bank_conflicts(mode, monkeypatch
     else:
         cfg = workloads.decode_bf16("cpu", batch=1, heads=128, pages_per_seq=8, topk=300, pad_frac=0.05)
     if mode != "first" and mode != "first_fp8":
-        monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1" if mode == "eight_wavefronts" else "2")
+        monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")
     harness.lds_profile_start()
     try:
         out, lse, rc = harness.forward(cfg, n_splits=2)
@@ -810,16 +916,16 @@ def test_gemm_kernels_address_lds_without_bank_conflicts():
         assert stats["read_tr"][0] > 500 and all(r == 1.0 for r in _bank_ratio(stats).values()), stats
 
 
-def test_work_per_unit_of_the_three_many_heads_kernels(monkeypatch):
+def test_work_per_unit_of_the_two_many_heads_kernels(monkeypatch):
     """What each design does per 16 tokens x 128 heads, counted on the code as it runs: the same
     matrix work, and the LDS and global -> LDS traffic the designs were made to differ in."""
     from flagtree_amd import workloads
     cfg = workloads.decode_bf16("cpu", batch=1, heads=128, pages_per_seq=40, topk=1024, pad_frac=0.0)
     units = 1024 * 128 / (16 * 128)
     got = {}
-    for name, mode in (("first", None), ("eight_wavefronts", "1"), ("wavefront_per_head_group", "2")):
+    for name, mode in (("first", None), ("wavefront_per_head_group", "1")):
         if mode:
-            monkeypatch.setenv("FLAGTREE_SMLA_WIDE", mode)
+            monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", mode)
         harness.work_counts()
         out, lse, rc = harness.forward(cfg, n_splits=1)
         assert rc == 0
@@ -827,8 +933,8 @@ def test_work_per_unit_of_the_three_many_heads_kernels(monkeypatch):
     for w in got.values():
         assert abs(w["mfma_flops"] - 2 * 16 * 128 * (576 + 512)) < 1.0          # 4.456 MFLOP, nothing computed twice
     kb = lambda name, key: round(got[name][key] / 1024, 1)       # (the page-table row's move adds a few bytes per unit)
-    assert kb("first", "dma_bytes") == 36.0 and kb("eight_wavefronts", "dma_bytes") == 18.0 and kb("wavefront_per_head_group", "dma_bytes") == 18.0
-    assert kb("first", "lds_read_bytes") == 144.0 and kb("eight_wavefronts", "lds_read_bytes") == 216.0
+    assert kb("first", "dma_bytes") == 36.0 and kb("wavefront_per_head_group", "dma_bytes") == 18.0
+    assert kb("first", "lds_read_bytes") == 144.0
     assert kb("wavefront_per_head_group", "lds_read_bytes") == 136.0 and got["wavefront_per_head_group"]["lds_write_bytes"] == 0.0
-    assert got["wavefront_per_head_group"]["barriers_x_waves"] < got["first"]["barriers_x_waves"] < got["eight_wavefronts"]["barriers_x_waves"]
+    assert got["wavefront_per_head_group"]["barriers_x_waves"] < got["first"]["barriers_x_waves"]
 

@@ -1,6 +1,6 @@
 """GPU parity of the kernel paths that have not been timed or run on hardware yet: the many-heads
 kernel over an fp8 cache (raw records by global -> LDS moves, converted LDS -> LDS) and the two
-opt-in second designs (FLAGTREE_SMLA_FEW_FP8, FLAGTREE_SMLA_WIDE) and the opt-in token order
+opt-in second designs (FLAGTREE_SMLA_FEW_FP8, FLAGTREE_SMLA_HEAD_GROUPS) and the opt-in token order
 (FLAGTREE_SMLA_TOKEN_BANDS).  The file sorts after the other
 GPU test files on purpose: under `pytest -x` a failure here cannot hide the results of the paths
 the defaults rest on.  Same bars: out max-abs <= 1e-2, lse <= 1e-3 against the float64 oracle."""
@@ -53,9 +53,9 @@ def test_logit_cap_many_heads_fp8(dev, splits):
 @pytest.mark.parametrize("topk,n_splits,heads", [(1, 1, 40), (33, 1, 128), (64, 2, 65), (97, 1, 128), (129, 2, 128), (200, 3, 128),
                                                  (1030, 1, 40), (2100, 2, 128), (2048, None, 128)])
 def test_head_group_kernel_fp8_pipeline(dev, monkeypatch, topk, n_splits, heads):
-    """The raw-record pipeline inside the wavefront-per-head-group kernel (FLAGTREE_SMLA_WIDE=2)."""
+    """The raw-record pipeline inside the wavefront-per-head-group kernel (FLAGTREE_SMLA_HEAD_GROUPS=1)."""
     from flagtree_amd import workloads
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "2")
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")
     cfg = workloads.decode_fp8(dev, batch=3, heads=heads, pages_per_seq=40, topk=topk, pad_frac=0.0 if topk < 40 else 0.04)
     out, lse = _fwd(cfg, n_splits=n_splits)
     _check(cfg, out, lse)
@@ -147,9 +147,9 @@ def test_column_split_fp8_kernel_edge_cases_and_dense(dev, few_fp8_kernel):
 
 # ---- the 128-heads-per-workgroup bf16 kernel (opt-in until it has been measured) ----------------
 
-@pytest.fixture(params=["1", "2"], ids=["eight_wavefronts", "wavefront_per_head_group"])
-def wide_kernel(request, monkeypatch):
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", request.param)
+@pytest.fixture
+def wide_kernel(monkeypatch):
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")
 
 
 @pytest.mark.parametrize("heads,n_splits,topk", [(128, 1, 512), (128, 2, 512), (64, 3, 300), (200, 2, 700), (128, None, 2048),
@@ -161,14 +161,13 @@ def test_128_heads_kernel_against_oracle(dev, wide_kernel, heads, n_splits, topk
     _check(cfg, out, lse)
 
 
-@pytest.mark.parametrize("mode", ["1", "2"])
-def test_128_heads_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch, mode):
+def test_128_heads_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch):
     """Headline decode size: the two kernels agree to the bar (they sum in different orders), and a
     slice of the batch agrees with the oracle."""
     from flagtree_amd import workloads
     cfg = workloads.decode_bf16(dev)
     out0, lse0 = _fwd(cfg)
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", mode)
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")
     out1, lse1 = _fwd(cfg)
     torch.cuda.synchronize()
     assert not torch.equal(out0, out1)                       # it really is the other kernel

@@ -3,7 +3,8 @@ handed to each lane, tests/hw_model/primitives.hip) and compared bit for bit wit
 emulator's model of it and with the documented behaviour stated in numpy.  A kernel test that
 passes on the emulator and fails on the GPU points here first: either a primitive differs (this
 file names it) or the fault is in what the emulator does not model (registers, timing, caches).
-The file sorts after the kernel parity tests: the probes themselves are new to the hardware."""
+tests/conftest.py moves the probes to the front of a GPU run (seconds, and their output is what
+sorts a later failure); the whole-kernel comparisons below run where the file name sorts: last."""
 import os
 import sys
 
@@ -53,7 +54,16 @@ def test_primitive_on_the_gpu_matches_the_emulator_and_the_documentation(dev, gp
     got = run_on_gpu(gpu_probes, dev, name, rec)
     against_emulator = cases.differences(name, got, run_on_emulator(name, rec))
     against_documentation = cases.differences(name, got, cases.expect(name, rec))
-    assert not against_emulator and not against_documentation, (against_emulator, against_documentation)
+    if against_emulator or against_documentation:
+        # A probe is a diagnostic of the test models, not of the product: it must not end a run
+        # started with -x before the parity tests have had their turn.  The mismatch is printed
+        # now, recorded, and fails the last test of this file.
+        _MISMATCHES.append((name, seed, against_emulator, against_documentation))
+        print(f"PROBE MISMATCH {name} seed {seed}: emulator {against_emulator} documentation {against_documentation}", flush=True)
+        pytest.xfail(f"probe {name} differs from its model (reported by the last test of this file)")
+
+
+_MISMATCHES = []
 
 
 # ---- whole kernels: the GPU against the emulator -----------------------------------------------
@@ -69,7 +79,7 @@ def _to_device(cfg, dev):
 
 
 @pytest.mark.parametrize("n_splits", [1, 3])
-@pytest.mark.parametrize("kernel", ["many_heads_bf16", "many_heads_fp8", "eight_wavefronts_bf16", "wavefront_per_head_group_bf16",
+@pytest.mark.parametrize("kernel", ["many_heads_bf16", "many_heads_fp8", "wavefront_per_head_group_bf16",
                                     "wavefront_per_head_group_fp8", "few_heads_bf16", "few_heads_fp8", "few_heads_fp8_column_split"])
 def test_kernel_on_the_gpu_stays_within_rounding_of_the_emulator(dev, gpu_probes, monkeypatch, kernel, n_splits):
     import numpy as np
@@ -78,7 +88,7 @@ def test_kernel_on_the_gpu_stays_within_rounding_of_the_emulator(dev, gpu_probes
     from test_gpu_sparse_mla import _fwd
     from _util import to_np
     heads = 16 if kernel.startswith("few_heads") else 128
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1" if kernel.startswith("eight") else ("2" if kernel.startswith("wavefront") else "0"))
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel.startswith("wavefront") else "0")
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel.endswith("column_split") else "0")
     if "fp8" in kernel:
         cfg, _ = _fp8_cfg(3, heads, 12, 330, pad_frac=0.05)
@@ -95,3 +105,8 @@ def test_kernel_on_the_gpu_stays_within_rounding_of_the_emulator(dev, gpu_probes
     le, lg = to_np(lse_e).reshape(-1, heads), to_np(lse_g).reshape(-1, heads)
     assert np.abs(lg - le).max() <= 2e-5, np.abs(lg - le).max()
     assert (np.abs(og - oe) <= 2.0 ** -7 * np.abs(oe) + 1e-6).all(), np.abs(og - oe).max()       # two bf16 steps
+
+
+def test_every_primitive_matched_its_model(dev, gpu_probes):
+    """Collected last of all GPU tests: the probes at the front of the run only record a mismatch."""
+    assert not _MISMATCHES, _MISMATCHES

@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
         assert hasattr(lib, n), f"{n} declared in include/flagtree_smla.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.smla_abi_version() == 2
+    assert lib.smla_abi_version() == 3
 
 
 def test_status_texts(lib):
@@ -119,16 +119,14 @@ def test_split_planning_follows_the_kernel_switches(lib, monkeypatch):
     device with, so the planner doubles the splits; the switches are read at every call.
     (Without a GPU the library plans for 256 compute units.)"""
     BF16, FP8 = 0, 1
-    monkeypatch.delenv("FLAGTREE_SMLA_WIDE", raising=False)
+    monkeypatch.delenv("FLAGTREE_SMLA_HEAD_GROUPS", raising=False)
     monkeypatch.delenv("FLAGTREE_SMLA_FEW_FP8", raising=False)
     base = [lib.smla_plan_splits(BF16, 64, 128, 2048), lib.smla_plan_splits(FP8, 64, 128, 2048), lib.smla_plan_splits(FP8, 128, 16, 2048)]
     assert base == [2, 2, 2]
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "1")                 # eight wavefronts: bf16 caches only
-    assert [lib.smla_plan_splits(BF16, 64, 128, 2048), lib.smla_plan_splits(FP8, 64, 128, 2048)] == [4, 2]
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "2")                 # a wavefront per head group: both formats
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")          # a wavefront per head group: both formats
     assert [lib.smla_plan_splits(BF16, 64, 128, 2048), lib.smla_plan_splits(FP8, 64, 128, 2048)] == [4, 4]
     assert lib.smla_plan_splits(FP8, 128, 16, 2048) == 2           # few heads: not its business
-    monkeypatch.setenv("FLAGTREE_SMLA_WIDE", "0")
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "0")
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")              # two workgroups per compute unit
     assert lib.smla_plan_splits(FP8, 128, 16, 2048) == 4 and lib.smla_plan_splits(BF16, 64, 128, 2048) == 2
 

@@ -17,11 +17,9 @@ LDS_PER_CU = 160 * 1024
 # Kernels that may park registers in scratch memory OUTSIDE their inner loops (checked below):
 #  * the two-workgroups-per-CU fp8 kernel is capped at 256 registers and parks a few across the
 #    per-chunk set-up.
-#  * the 128-heads-per-workgroup kernel keeps 200 of its 256 registers for Q and accumulators; it
-#    parks values across the per-chunk set-up and while the accumulators drain in the epilogue.
 #  * the wavefront-per-head-group kernel holds 144 Q and 256 accumulator registers; it parks values
 #    across the per-chunk set-up and in the epilogue's merge.
-MAY_SPILL = ("fwd_few_fp8_kernel", "fwd_wide_kernel", "fwd_group_kernel")
+MAY_SPILL = ("fwd_few_fp8_kernel", "fwd_group_kernel")
 
 _cache = {}
 
@@ -113,12 +111,6 @@ def test_two_workgroups_of_the_column_split_fp8_kernel_fit_a_cu():
     few = _resource_usage("smla_mfma_few_fp8.hip")
     assert few and all(u["Occupancy"] >= 2 and u["LDS Size"] <= LDS_PER_CU // 2 and u["VGPRs"] + u["AGPRs"] <= 256
                        for u in few.values()), few
-
-
-def test_two_wavefronts_per_simd_of_the_128_heads_kernel():
-    wide = _resource_usage("smla_mfma_wide.hip")
-    assert wide and all(u["Occupancy"] == 2 and u["VGPRs"] + u["AGPRs"] <= 256 and u["LDS Size"] <= LDS_PER_CU
-                        for u in wide.values()), wide
 
 
 def test_one_wavefront_per_simd_kernels_use_the_whole_register_file():
