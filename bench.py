@@ -48,6 +48,9 @@ def parse():
                          "FLAGTREE_SMLA_HEAD_GROUPS=1; opt-in until measured)")
     ap.add_argument("--few-fp8", action="store_true",
                     help="decode_fp8 on the two-workgroups-per-CU kernel (sets FLAGTREE_SMLA_FEW_FP8=1; opt-in until measured)")
+    ap.add_argument("--fp8-mfma", action="store_true",
+                    help="decode_fp8 on the kernel that contracts the records' e4m3 codes with fp8 MFMAs (sets "
+                         "FLAGTREE_SMLA_FP8_MFMA=1; opt-in until measured)")
     ap.add_argument("--token-bands", action="store_true",
                     help="each XCD takes a contiguous band of tokens instead of every eighth one (sets "
                          "FLAGTREE_SMLA_TOKEN_BANDS=1; for prefill_causal_bf16; opt-in until measured)")
@@ -138,6 +141,8 @@ def main():
         sys.exit(2)
     if a.few_fp8:
         os.environ["FLAGTREE_SMLA_FEW_FP8"] = "1"
+    if a.fp8_mfma:
+        os.environ["FLAGTREE_SMLA_FP8_MFMA"] = "1"
     if a.head_groups:
         os.environ["FLAGTREE_SMLA_HEAD_GROUPS"] = "1"
     if a.token_bands:
@@ -272,9 +277,9 @@ def main():
         roof = dict(bound="mfma", achieved=flops / (kern_ms * 1e-3) / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
     # (the stored counter figures were taken on the default kernels: none for a kernel behind a switch)
-    roof["traffic"] = None if (a.head_groups or a.few_fp8 or a.token_bands) else measured_traffic(a.workload)
+    roof["traffic"] = None if (a.head_groups or a.few_fp8 or a.fp8_mfma or a.token_bands) else measured_traffic(a.workload)
     roof["traffic_source"] = TRAFFIC_NOTE
-    roof["kernel"] = many_heads_kernel(a, fmt) if H > 32 else ("fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
+    roof["kernel"] = many_heads_kernel(a, fmt) if H > 32 else ("fwd_few_f8_kernel" if a.fp8_mfma and hbm_bound else "fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
     roof["kernel_ms"] = kern_ms
     roof["other_bound"] = (dict(bound="hbm", achieved=nbytes / (kern_ms * 1e-3) / 1e9, peak=PEAK_HBM_GBS, unit="GB/s")
                            if not hbm_bound else

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libflagtree_smla.so")
-SOURCES = ["smla_api.hip", "smla_scalar.hip", "smla_mfma_tall.hip", "smla_mfma_short.hip", "smla_mfma_few_fp8.hip", "smla_mfma_group.hip", "gemm_rs.hip", "topk_select.hip"]
+SOURCES = ["smla_api.hip", "smla_scalar.hip", "smla_mfma_tall.hip", "smla_mfma_short.hip", "smla_mfma_few_fp8.hip", "smla_mfma_few_f8.hip", "smla_mfma_group.hip", "gemm_rs.hip", "topk_select.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

@@ -40,6 +40,14 @@ bool few_fp8_enabled() {
   return e != nullptr && e[0] == '1';
 }
 
+// FLAGTREE_SMLA_FP8_MFMA=1 sends few-heads launches over an fp8 cache to the kernel that contracts
+// the records' e4m3 codes on the matrix cores as they are (smla_mfma_few_f8.hip; also two
+// workgroups per CU).  It wins over FLAGTREE_SMLA_FEW_FP8.
+bool fp8_mfma_enabled() {
+  const char* e = getenv("FLAGTREE_SMLA_FP8_MFMA");
+  return e != nullptr && e[0] == '1';
+}
+
 // FLAGTREE_SMLA_TOKEN_BANDS=1 gives each XCD a contiguous band of tokens instead of every eighth
 // token (for causal prefill; see token_of).
 bool token_bands_enabled() {
@@ -144,7 +152,7 @@ int smla_plan_splits(int kv_format, int32_t n_tokens, int32_t n_heads, int32_t t
   // one 4-wave workgroup per CU is resident at a time; each covers 64 (or, for <= 32 heads, 16)
   // heads of one token
   // (the opt-in fp8 kernel keeps two workgroups per CU; every further split adds a partial to publish and fold)
-  const bool few_fp8 = kv_format == SMLA_KV_FP8_B128 && n_heads <= 32 && few_fp8_enabled();
+  const bool few_fp8 = kv_format == SMLA_KV_FP8_B128 && n_heads <= 32 && (few_fp8_enabled() || fp8_mfma_enabled());
   const int slots = few_fp8 ? 2 * device_cus() : device_cus();
   const bool wide = n_heads > 32 && head_groups_enabled();
   const int per_wg = n_heads <= 32 ? 16 : (wide ? 128 : 64);
@@ -222,6 +230,7 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
   }
   if (n_heads > 32 && head_groups_enabled()) rc = launch_fwd_group(kv_format, p, s);
   else if (n_heads > 32) rc = launch_fwd_tall(kv_format, p, s);
+  else if (kv_format == SMLA_KV_FP8_B128 && fp8_mfma_enabled()) rc = launch_fwd_few_f8(p, s);
   else if (kv_format == SMLA_KV_FP8_B128 && few_fp8_enabled()) rc = launch_fwd_few_fp8(p, s);
   else rc = launch_fwd_short(kv_format, p, s);
   if (rc != SMLA_OK || n_splits == 1 || p.merge_in_launch) return rc;

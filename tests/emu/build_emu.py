@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 CSRC = os.path.join(ROOT, "flagtree_amd", "csrc")
 LIB_PATH = os.path.join(HERE, "libflagtree_smla_emu.so")
-SOURCES = ["smla_api.hip", "smla_scalar.hip", "smla_mfma_tall.hip", "smla_mfma_short.hip", "smla_mfma_few_fp8.hip", "smla_mfma_group.hip", "gemm_rs.hip", "topk_select.hip"]
+SOURCES = ["smla_api.hip", "smla_scalar.hip", "smla_mfma_tall.hip", "smla_mfma_short.hip", "smla_mfma_few_fp8.hip", "smla_mfma_few_f8.hip", "smla_mfma_group.hip", "gemm_rs.hip", "topk_select.hip"]
 HW_MODEL = os.path.join(os.path.dirname(HERE), "hw_model")      # probes of single instructions, built for both sides
 CXX = os.environ.get("EMU_CXX", "/opt/rocm/llvm/bin/clang++")
 FLAGS = ["-x", "c++", "-std=c++17", "-O2", "-g1", "-fPIC", "-ffp-contract=off", "-fno-strict-aliasing",

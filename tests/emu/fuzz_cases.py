@@ -24,7 +24,8 @@ import oracle           # noqa: E402
 from _util import max_abs, oracle_inputs, to_np   # noqa: E402
 
 G = harness.Guarded
-SWITCHES = ("FLAGTREE_SMLA_FEW_FP8", "FLAGTREE_SMLA_HEAD_GROUPS", "FLAGTREE_SMLA_TOKEN_BANDS", "FLAGTREE_SMLA_SEPARATE_MERGE")
+SWITCHES = ("FLAGTREE_SMLA_FEW_FP8", "FLAGTREE_SMLA_FP8_MFMA", "FLAGTREE_SMLA_HEAD_GROUPS", "FLAGTREE_SMLA_TOKEN_BANDS",
+            "FLAGTREE_SMLA_SEPARATE_MERGE")
 
 
 def random_schedule(rng):
@@ -53,7 +54,7 @@ def forward_case(seed):
     for k in SWITCHES:
         os.environ.pop(k, None)
     if rng.random() < 0.5:                                  # the opt-in kernels (each applies to its own head counts)
-        os.environ["FLAGTREE_SMLA_FEW_FP8"] = "1"
+        os.environ["FLAGTREE_SMLA_FP8_MFMA" if rng.random() < 0.5 else "FLAGTREE_SMLA_FEW_FP8"] = "1"
         os.environ["FLAGTREE_SMLA_HEAD_GROUPS"] = "1"
     if rng.random() < 0.5:
         os.environ["FLAGTREE_SMLA_TOKEN_BANDS"] = "1"

@@ -283,7 +283,77 @@ inline Acc mfma(Frag a, Frag b, Acc c, uint32_t tag) {
   }
   return d;
 }
+
+// D = A . B + C, 16 x 16 x (4 * BYTES), over fp8 (e4m3fn) operands.  Lane m + 16 g holds BYTES
+// values of row m of A (of column n of B).  Which k a (g, byte) pair stands for is the same
+// function for A and for B, so the sum over all pairs does not depend on it, and neither does a
+// kernel that loads both operands by the same rule.  Products of two e4m3 values are exact in
+// fp32; they are summed in fp32 (the hardware's order is its own: results agree to rounding).
+// `scaled`: each operand is multiplied by 2^(e - 127), e its lane's scale byte; the model holds
+// for scale bytes that are the same in every lane (which lane's byte serves which block of k is
+// then immaterial) and refuses anything else.
+typedef __attribute__((ext_vector_type(8))) int v8i;
+template <int BYTES, typename Frag>
+inline v4f mfma16_fp8(Frag a, Frag b, v4f c, bool scaled, uint32_t scale_a, uint32_t scale_b, uint32_t tag) {
+  static_assert(sizeof(Frag) == BYTES, "fragment = BYTES fp8 values");
+  struct Post { Frag a, b; uint32_t sa, sb; } post{a, b, scale_a & 0xffu, scale_b & 0xffu};
+  count_mfma(16, 4 * BYTES);
+  const int par = wave_rendezvous(&post, sizeof(post), tag);
+  const int l = self()->lane, n = l % 16;
+  float factor = 1.f;
+  if (scaled) {
+    for (int src = 0; src < 64; ++src) {
+      if (!wave_lane_live(src)) continue;
+      Post other;
+      memcpy(&other, wave_slot(par, src), sizeof(other));
+      if (other.sa != post.sa || other.sb != post.sb) fail("scaled fp8 MFMA with scale bytes that differ between lanes: not modelled");
+    }
+    factor = ldexpf(1.f, (int)post.sa - 127 + (int)post.sb - 127);
+  }
+  float bcol[4 * BYTES];
+  for (int g = 0; g < 4; ++g) {
+    uint8_t bytes[BYTES];
+    memcpy(bytes, wave_slot(par, n + 16 * g) + offsetof(Post, b), BYTES);
+    for (int j = 0; j < BYTES; ++j) bcol[g * BYTES + j] = e4m3fn_to_f32(bytes[j]);
+  }
+  v4f d = c;
+  for (int r = 0; r < 4; ++r) {
+    const int m = 4 * (l / 16) + r;
+    float sum = 0.f;
+    for (int g = 0; g < 4; ++g) {
+      uint8_t bytes[BYTES];
+      memcpy(bytes, wave_slot(par, m + 16 * g), BYTES);
+      for (int j = 0; j < BYTES; ++j) sum += e4m3fn_to_f32(bytes[j]) * bcol[g * BYTES + j];
+    }
+    d[r] = c[r] + factor * sum;
+  }
+  return d;
+}
+inline v4f mfma_scale_16x16x128_f8f6f4(v8i a, v8i b, v4f c, int cbsz, int blgp, int opsel_a, int scale_a, int opsel_b, int scale_b) {
+  if (cbsz != 0 || blgp != 0) fail("scaled MFMA: only e4m3 operands (cbsz = blgp = 0) are modelled");
+  return mfma16_fp8<32, v8i>(a, b, c, true, (uint32_t)scale_a >> (8 * (opsel_a & 3)), (uint32_t)scale_b >> (8 * (opsel_b & 3)), 0x4d463830u);
+}
+// v_perm_b32: byte i of the result is byte sel[i] of the 8 bytes {b = bytes 0..3, a = bytes 4..7};
+// selector 0x0c gives 0x00.  (The sign-replicating selectors 8 .. 11 and 0x0d .. are not modelled.)
+inline uint32_t perm_b32(uint32_t a, uint32_t b, uint32_t sel) {
+  const uint64_t both = ((uint64_t)a << 32) | b;
+  uint32_t out = 0;
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t s = (sel >> (8 * i)) & 0xffu;
+    uint32_t byte;
+    if (s < 8) byte = (uint32_t)(both >> (8 * s)) & 0xffu;
+    else if (s == 0x0c) byte = 0;
+    else fail("v_perm_b32 selector %u is not modelled", s);
+    out |= byte << (8 * i);
+  }
+  return out;
+}
 }  // namespace emu
+#define __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, b, c, x, y, z) \
+  emu::mfma16_fp8<8, long>((a), (b), (c), false, 127u, 127u, 0x4d463833u)
+#define __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, cbsz, blgp, opa, sa, opb, sb) \
+  emu::mfma_scale_16x16x128_f8f6f4((a), (b), (c), (cbsz), (blgp), (opa), (sa), (opb), (sb))
+#define __builtin_amdgcn_perm(a, b, sel) emu::perm_b32((a), (b), (sel))
 #define __builtin_amdgcn_cvt_pk_f32_fp8(w, hi) emu::cvt_pk_f32_fp8((w), (hi))
 #define __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, s, hi) emu::cvt_scalef32_pk_bf16_fp8((w), (s), (hi))
 #define __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, hi) emu::cvt_pk_fp8_f32((a), (b), (old), (hi))

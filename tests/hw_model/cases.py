@@ -53,7 +53,14 @@ def make_input(name, seed):
     u32 = rec.view(np.uint32)
     f32 = rec.view(np.float32)
     u16 = rec.view(np.uint16)
-    if name.startswith("MFMA"):
+    if name in ("MFMA_16X16X32_FP8", "MFMA_SCALE_16X16X128_FP8"):
+        # e4m3 codes of small integers: every product and partial sum is exact in fp32, whatever the order
+        import oracle
+        n_ab = 16 if name == "MFMA_16X16X32_FP8" else 64
+        rec[:, :n_ab] = oracle.e4m3_encode(g.integers(-4, 5, size=(LANES, n_ab)).astype(np.float32))
+        c0 = n_ab // 4
+        f32[:, c0:c0 + 4] = g.integers(-8, 9, size=(LANES, 4)).astype(np.float32)
+    elif name.startswith("MFMA"):
         # small integers: every product and every partial sum is exact in fp32, whatever the order
         n_ab = 8 if name == "MFMA_16X16X16_BF16" else 16
         u16[:, :n_ab] = bf16_bits(g.integers(-4, 5, size=(LANES, n_ab)).astype(np.float32))
@@ -110,6 +117,23 @@ def expect(name, rec):
         for lane in range(LANES):                     # C/D: lane holds column lane % 16, rows 4 * (lane // 16) + 0..3
             for r in range(4):
                 of32[lane, r] = d[4 * (lane // 16) + r, lane % 16] + f32[lane, c0 + r]
+    elif name in ("MFMA_16X16X32_FP8", "MFMA_SCALE_16X16X128_FP8"):
+        # Lane m + 16 g holds `nb` values of row m of A and, behind them, of column m of B.  A (g, byte)
+        # pair stands for the same k in both operands, so the sum over all pairs is the product
+        # whatever that k is.  The scaled form multiplies by 2^(127 - 127) * 2^(123 - 127).
+        import oracle
+        nb = 8 if name == "MFMA_16X16X32_FP8" else 32
+        a = oracle.e4m3_decode(rec[:, :nb]).astype(np.float64).reshape(4, 16, nb)          # [g, m, byte]
+        b = oracle.e4m3_decode(rec[:, nb:2 * nb]).astype(np.float64).reshape(4, 16, nb)     # [g, n, byte]
+        d = np.einsum("gmj,gnj->mn", a, b) * (1.0 if name == "MFMA_16X16X32_FP8" else 2.0 ** -4)
+        c0 = nb // 2
+        for lane in range(LANES):
+            for r in range(4):
+                of32[lane, r] = d[4 * (lane // 16) + r, lane % 16] + f32[lane, c0 + r]
+    elif name == "BYTE_PERMUTE":
+        both = rec[:, [4, 5, 6, 7, 0, 1, 2, 3]]           # bytes 0..3 = b (the second operand), 4..7 = a
+        out[:, 0:4] = both[:, [0, 2, 4, 6]]
+        out[:, 4:8] = both[:, [1, 3, 5, 7]]
     elif name == "MFMA_32X32X16_BF16":
         a, b = _mfma_operands(rec, 32, 16, 8)
         d = a @ b

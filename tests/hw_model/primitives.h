@@ -19,7 +19,10 @@ enum {
   HWM_COMPARE_AND_SHIFT_IN = 10,   /* in: x, y, mask (u32);  out: mask after shift_in_gt, after shift_in_eq */
   HWM_AGENT_SCOPE_ACCESSES = 11,   /* in: 16 B at 0 (stored), 16 B at 16 (loaded);  out: both */
   HWM_APPROXIMATE_FUNCTIONS = 12,  /* in: 4 floats;  out: exp2, log2(|x| + 1e-3), 1 / (|x| + 1e-3) of each */
-  HWM_COUNT = 13
+  HWM_MFMA_16X16X32_FP8 = 13,      /* in: A 8 B, B 8 B, C 16 B at 0/8/16 (e4m3 codes);  out: D 16 B */
+  HWM_MFMA_SCALE_16X16X128_FP8 = 14, /* in: A 32 B, B 32 B, C 16 B at 0/32/64; scale bytes 127 (A) and 123 (B) in every lane;  out: D 16 B */
+  HWM_BYTE_PERMUTE = 15,           /* in: a, b (u32);  out: v_perm_b32 with the two selectors the fp8 V operand is put together with */
+  HWM_COUNT = 16
 };
 
 #ifdef __cplusplus

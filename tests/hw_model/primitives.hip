@@ -24,6 +24,7 @@ using namespace smla::hw;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
 
 constexpr int kRecord = HWM_RECORD_BYTES;
 constexpr int kLanes = HWM_LANES;
@@ -116,6 +117,16 @@ __global__ __launch_bounds__(64) void probe_kernel(const uint8_t* __restrict__ i
     store_b128_agent(reinterpret_cast<float*>(o), get<f32x4>(r));
     const buffer_rsrc rsrc = make_rsrc(in);
     put<f32x4>(o + 16, load_b128_agent(rsrc, (uint32_t)(kRecord * lane + 16)));
+  } else if constexpr (W == HWM_MFMA_16X16X32_FP8) {
+    put<f32x4>(o, __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(get<long>(r), get<long>(r + 8), get<f32x4>(r + 16), 0, 0, 0));
+  } else if constexpr (W == HWM_MFMA_SCALE_16X16X128_FP8) {
+    // e4m3 operands (format codes 0), scale bytes 2^0 for A and 2^-4 for B, the same in every lane and every byte
+    put<f32x4>(o, __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(get<i32x8>(r), get<i32x8>(r + 32), get<f32x4>(r + 64), 0, 0,
+                                                                  0, 0x7f7f7f7f, 0, 0x7b7b7b7b));
+  } else if constexpr (W == HWM_BYTE_PERMUTE) {
+    const uint32_t a = get<uint32_t>(r), b = get<uint32_t>(r + 4);
+    put<uint32_t>(o, __builtin_amdgcn_perm(a, b, 0x06040200u));
+    put<uint32_t>(o + 4, __builtin_amdgcn_perm(a, b, 0x07050301u));
   } else if constexpr (W == HWM_APPROXIMATE_FUNCTIONS) {
     float* d = reinterpret_cast<float*>(o);
 #pragma unroll
@@ -153,6 +164,9 @@ extern "C" int hwm_run(int which, const void* in, void* out, void* stream) {
     case HWM_COMPARE_AND_SHIFT_IN: return launch<HWM_COMPARE_AND_SHIFT_IN>(in, out, s);
     case HWM_AGENT_SCOPE_ACCESSES: return launch<HWM_AGENT_SCOPE_ACCESSES>(in, out, s);
     case HWM_APPROXIMATE_FUNCTIONS: return launch<HWM_APPROXIMATE_FUNCTIONS>(in, out, s);
+    case HWM_MFMA_16X16X32_FP8: return launch<HWM_MFMA_16X16X32_FP8>(in, out, s);
+    case HWM_MFMA_SCALE_16X16X128_FP8: return launch<HWM_MFMA_SCALE_16X16X128_FP8>(in, out, s);
+    case HWM_BYTE_PERMUTE: return launch<HWM_BYTE_PERMUTE>(in, out, s);
     default: return -3;
   }
 }

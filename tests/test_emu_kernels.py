@@ -253,10 +253,16 @@ def test_128_heads_kernel_edge_cases_redo_prefill_and_dense(wide_kernel):
         assert max_abs(to_np(lse), wl) <= LSE_TOL and max_abs(to_np(out), wo) <= OUT_TOL
 
 
-@pytest.fixture
-def few_fp8_kernel(monkeypatch):
-    """Routes few-heads fp8 launches to the two-workgroups-per-CU kernel (opt-in until it is measured)."""
-    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
+FEW_HEADS_FP8_SWITCHES = {"column_split": "FLAGTREE_SMLA_FEW_FP8", "fp8_mfma": "FLAGTREE_SMLA_FP8_MFMA"}
+
+
+@pytest.fixture(params=["column_split", "fp8_mfma"])
+def few_fp8_kernel(request, monkeypatch):
+    """Routes few-heads fp8 launches to one of the two-workgroups-per-CU kernels (opt-in until they are
+    measured): the column-split one that converts records to bf16, or the one that contracts the
+    records' e4m3 codes on the matrix cores."""
+    monkeypatch.setenv(FEW_HEADS_FP8_SWITCHES[request.param], "1")
+    return FEW_HEADS_FP8_SWITCHES[request.param]
 
 
 @pytest.mark.parametrize("heads,n_splits,topk", [(16, 1, 300), (16, 2, 300), (8, 1, 70), (16, 3, 1100), (30, 2, 200), (16, 4, 40)])
@@ -265,7 +271,7 @@ def test_fp8_records_column_split_kernel(few_fp8_kernel, heads, n_splits, topk):
     out, lse = _forward_all_ways(cfg, n_splits)
     _check(cfg, out, lse)
     # it is a different kernel: same results to the bar, not to the bit
-    os.environ.pop("FLAGTREE_SMLA_FEW_FP8")
+    os.environ.pop(few_fp8_kernel)
     out1, lse1, rc = harness.forward(cfg, n_splits=n_splits)
     assert rc == 0 and not torch.equal(out1.view(torch.int16), out.view(torch.int16))
     assert max_abs(to_np(out1), to_np(out)) <= 2e-3 and max_abs(to_np(lse1), to_np(lse)) <= 1e-5
@@ -457,7 +463,7 @@ def test_dense_decode_with_logit_cap(heads, fmt, std, cap, min_diff):
 
 
 @pytest.mark.parametrize("seed", list(range(12)))
-@pytest.mark.parametrize("few_fp8", [False, True, "head_groups"])
+@pytest.mark.parametrize("few_fp8", [False, True, "fp8_mfma", "head_groups"])
 def test_random_shapes_against_oracle(seed, few_fp8, monkeypatch):
     """Seeded draws over head counts, list lengths, page sizes, tokens per sequence, split counts,
     padding patterns, page tables with holes and both cache formats (the GPU suite's recipe at sizes
@@ -480,7 +486,7 @@ def test_random_shapes_against_oracle(seed, few_fp8, monkeypatch):
     elif few_fp8:
         if fmt != "fp8_e4m3_b128" or heads > 32:
             pytest.skip("the opt-in kernel covers few heads over an fp8 cache")
-        monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
+        monkeypatch.setenv("FLAGTREE_SMLA_FP8_MFMA" if few_fp8 == "fp8_mfma" else "FLAGTREE_SMLA_FEW_FP8", "1")
     if paged:
         pages_per_seq = -(-ctx // page_size)
         n_pages = batch * pages_per_seq + 3
@@ -546,7 +552,7 @@ def _header(ws):
     return ws[_lib.SMLA_WS_HEADER_OFFSET:_lib.SMLA_WS_HEADER_OFFSET + 16].view(torch.int32)
 
 
-@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split"])
+@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split", "few_heads_fp8_mfma"])
 def test_merging_workgroup_really_waits_for_the_others(kernel, monkeypatch):
     """With one workgroup at a time the last arrival of a split merge always finds the others'
     partials published.  Here several share the machine and are switched every few steps: the
@@ -556,7 +562,8 @@ def test_merging_workgroup_really_waits_for_the_others(kernel, monkeypatch):
     heads = 128 if kernel in ("many_heads", "wavefront_per_head_group") else 16
     monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel == "wavefront_per_head_group" else "0")
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel == "few_heads_fp8_column_split" else "0")
-    if kernel == "few_heads_fp8_column_split":
+    monkeypatch.setenv("FLAGTREE_SMLA_FP8_MFMA", "1" if kernel == "few_heads_fp8_mfma" else "0")
+    if kernel.startswith("few_heads_fp8"):
         cfg, _ = _fp8_cfg(3, heads, 20, 400, pad_frac=0.05)
     else:
         cfg = workloads.decode_bf16("cpu", batch=3, heads=heads, pages_per_seq=20, topk=400, pad_frac=0.05)
@@ -610,7 +617,7 @@ def test_stale_arrival_word_is_flagged_not_hung(heads, stale, schedule):
     assert max_abs(to_np(lse2), to_np(ref_lse)) <= 1e-3 and max_abs(to_np(out2), to_np(ref_out)) <= 1e-2
 
 
-@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split"])
+@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split", "few_heads_fp8_mfma"])
 def test_flagged_workspace_stays_loud_until_the_host_has_looked(kernel, monkeypatch):
     """A launch that gave up may leave an arrival word in a state the next launch cannot tell from
     a legal one: here one ticket and the OTHER split's published bit, with two splits.  Judged by
@@ -621,7 +628,8 @@ def test_flagged_workspace_stays_loud_until_the_host_has_looked(kernel, monkeypa
     heads = 128 if kernel in ("many_heads", "wavefront_per_head_group") else 16
     monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel == "wavefront_per_head_group" else "0")
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel == "few_heads_fp8_column_split" else "0")
-    if kernel == "few_heads_fp8_column_split":
+    monkeypatch.setenv("FLAGTREE_SMLA_FP8_MFMA", "1" if kernel == "few_heads_fp8_mfma" else "0")
+    if kernel.startswith("few_heads_fp8"):
         cfg, _ = _fp8_cfg(2, heads, 6, 260, pad_frac=0.05)
     else:
         cfg = workloads.decode_bf16("cpu", batch=2, heads=heads, pages_per_seq=6, topk=260, pad_frac=0.05)
@@ -644,7 +652,7 @@ def test_flagged_workspace_stays_loud_until_the_host_has_looked(kernel, monkeypa
 
 
 @pytest.mark.parametrize("how", ["compute units of an unknown layout", "environment"])
-@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split"])
+@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group", "few_heads", "few_heads_fp8_column_split", "few_heads_fp8_mfma"])
 def test_splits_merged_by_a_second_launch(kernel, how, monkeypatch, schedule):
     """The merge inside the launch needs all workgroups of a token behind one L2, which the library
     only claims for compute-unit counts it knows the XCD layout of.  Elsewhere (here: 48 compute
@@ -654,7 +662,8 @@ def test_splits_merged_by_a_second_launch(kernel, how, monkeypatch, schedule):
     heads = 128 if kernel in ("many_heads", "wavefront_per_head_group") else 16
     monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel == "wavefront_per_head_group" else "0")
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel == "few_heads_fp8_column_split" else "0")
-    if kernel == "few_heads_fp8_column_split":
+    monkeypatch.setenv("FLAGTREE_SMLA_FP8_MFMA", "1" if kernel == "few_heads_fp8_mfma" else "0")
+    if kernel.startswith("few_heads_fp8"):
         cfg, _ = _fp8_cfg(3, heads, 6, 330, pad_frac=0.05)
     else:
         cfg = workloads.decode_bf16("cpu", batch=3, heads=heads, pages_per_seq=6, topk=330, pad_frac=0.05)
@@ -895,6 +904,29 @@ def test_few_heads_kernels_transposing_reads_take_two_passes(monkeypatch):
             stats = harness.lds_profile_stop()
         assert rc == 0 and stats["read_tr"][0] > 100
         assert _bank_ratio(stats)["read_tr"] == 2.0, stats
+
+
+def test_fp8_mfma_kernel_addresses_lds_without_bank_conflicts(monkeypatch):
+    """Records lie in LDS back to back, 656 bytes apart (36 words modulo 64).  The 16-byte score
+    reads of 16 consecutive records fall on 16 different bank groups by themselves; the 8-byte
+    transposing reads of the V operand take every second record of 16 (the tokens' order inside
+    the operands is 0 2 4 6 1 3 5 7 for that reason) and are free of conflicts as well."""
+    monkeypatch.setenv("FLAGTREE_SMLA_FP8_MFMA", "1")
+    cfg = _fp8_cfg(1, 16, 8, 300, pad_frac=0.05)[0]
+    harness.lds_profile_start()
+    try:
+        out, lse, rc = harness.forward(cfg, n_splits=2)
+    finally:
+        stats = harness.lds_profile_stop()
+    assert rc == 0
+    _check(cfg, out, lse)
+    assert stats["read"][0] > 500 and stats["read_tr"][0] > 300, stats
+    ratio = _bank_ratio(stats)
+    assert ratio["read_tr"] == 1.0 and ratio["write"] == 1.0, stats
+    # Known and accepted: the eight 4-byte reads of a token's block scale per tile and wavefront
+    # (four addresses a wavefront, 16 lanes on each) put token groups 0 and 2, and 1 and 3, on the same
+    # bank, two passes instead of one; every 16-byte read is one pass.  Pinned so a change shows.
+    assert ratio["read"] == 1.2, stats
 
 
 def test_gemm_kernels_address_lds_without_bank_conflicts():

@@ -77,9 +77,14 @@ def test_fp8_many_heads_against_scalar_kernel_at_size(dev):
 
 # ---- the two-workgroups-per-CU fp8 kernel (opt-in until it has been measured) -------------------
 
-@pytest.fixture
-def few_fp8_kernel(monkeypatch):
-    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
+FEW_HEADS_FP8_SWITCHES = {"column_split": "FLAGTREE_SMLA_FEW_FP8", "fp8_mfma": "FLAGTREE_SMLA_FP8_MFMA"}
+
+
+@pytest.fixture(params=["column_split", "fp8_mfma"])
+def few_fp8_kernel(request, monkeypatch):
+    """One of the two opt-in few-heads fp8 kernels: the column-split one that converts records to
+    bf16, or the one that contracts the records' e4m3 codes on the matrix cores."""
+    monkeypatch.setenv(FEW_HEADS_FP8_SWITCHES[request.param], "1")
 
 
 @pytest.mark.parametrize("heads,n_splits,topk", [(16, 1, 512), (16, 2, 512), (8, 3, 300), (30, 2, 700), (16, None, 2048)])
@@ -90,13 +95,14 @@ def test_column_split_fp8_kernel_against_oracle(dev, few_fp8_kernel, heads, n_sp
     _check(cfg, out, lse)
 
 
-def test_column_split_fp8_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch):
+@pytest.mark.parametrize("kernel", ["column_split", "fp8_mfma"])
+def test_column_split_fp8_kernel_against_the_first_kernel_at_full_size(dev, monkeypatch, kernel):
     """Full fp8 decode size: the two kernels agree to the bar (they sum in different orders), and a
     slice of the batch agrees with the oracle."""
     from flagtree_amd import workloads
     cfg = workloads.decode_fp8(dev)
     out0, lse0 = _fwd(cfg)
-    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")
+    monkeypatch.setenv(FEW_HEADS_FP8_SWITCHES[kernel], "1")
     out1, lse1 = _fwd(cfg)
     torch.cuda.synchronize()
     assert not torch.equal(out0, out1)                       # it really is the other kernel

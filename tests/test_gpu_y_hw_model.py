@@ -80,7 +80,7 @@ def _to_device(cfg, dev):
 
 @pytest.mark.parametrize("n_splits", [1, 3])
 @pytest.mark.parametrize("kernel", ["many_heads_bf16", "many_heads_fp8", "wavefront_per_head_group_bf16",
-                                    "wavefront_per_head_group_fp8", "few_heads_bf16", "few_heads_fp8", "few_heads_fp8_column_split"])
+                                    "wavefront_per_head_group_fp8", "few_heads_bf16", "few_heads_fp8", "few_heads_fp8_column_split", "few_heads_fp8_mfma"])
 def test_kernel_on_the_gpu_stays_within_rounding_of_the_emulator(dev, gpu_probes, monkeypatch, kernel, n_splits):
     import numpy as np
     from flagtree_amd import workloads
@@ -90,6 +90,7 @@ def test_kernel_on_the_gpu_stays_within_rounding_of_the_emulator(dev, gpu_probes
     heads = 16 if kernel.startswith("few_heads") else 128
     monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel.startswith("wavefront") else "0")
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1" if kernel.endswith("column_split") else "0")
+    monkeypatch.setenv("FLAGTREE_SMLA_FP8_MFMA", "1" if kernel.endswith("fp8_mfma") else "0")
     if "fp8" in kernel:
         cfg, _ = _fp8_cfg(3, heads, 12, 330, pad_frac=0.05)
     else:

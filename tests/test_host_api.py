@@ -121,6 +121,7 @@ def test_split_planning_follows_the_kernel_switches(lib, monkeypatch):
     BF16, FP8 = 0, 1
     monkeypatch.delenv("FLAGTREE_SMLA_HEAD_GROUPS", raising=False)
     monkeypatch.delenv("FLAGTREE_SMLA_FEW_FP8", raising=False)
+    monkeypatch.delenv("FLAGTREE_SMLA_FP8_MFMA", raising=False)
     base = [lib.smla_plan_splits(BF16, 64, 128, 2048), lib.smla_plan_splits(FP8, 64, 128, 2048), lib.smla_plan_splits(FP8, 128, 16, 2048)]
     assert base == [2, 2, 2]
     monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1")          # a wavefront per head group: both formats
@@ -129,6 +130,9 @@ def test_split_planning_follows_the_kernel_switches(lib, monkeypatch):
     monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "0")
     monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "1")              # two workgroups per compute unit
     assert lib.smla_plan_splits(FP8, 128, 16, 2048) == 4 and lib.smla_plan_splits(BF16, 64, 128, 2048) == 2
+    monkeypatch.setenv("FLAGTREE_SMLA_FEW_FP8", "0")
+    monkeypatch.setenv("FLAGTREE_SMLA_FP8_MFMA", "1")             # the fp8-MFMA kernel: two workgroups per compute unit as well
+    assert lib.smla_plan_splits(FP8, 128, 16, 2048) == 4 and lib.smla_plan_splits(BF16, 128, 16, 2048) == 2
 
 
 def test_python_surface_rejects_bad_input():

@@ -9,11 +9,13 @@ values, q bf16, 16 heads, top-k 2048.  Reference: the float64 oracle over the de
   q_split   a second pass over the residual: q ~ q_hi + q_lo / 16, both e4m3
   p_e4m3    probabilities (times the block scale) quantised to e4m3 per head for P.V
   p_split   the same in two e4m3 terms
-What it shows, and why the kernels still convert: one pass is far inside the bars on the benchmark's
-inputs, but breaks the LSE bar once scores are an order of magnitude larger or the attention is
-concentrated on a few rows; two passes restore it.  So the fp8 contraction has to be the two-pass
-form (2 x the QK matrix work at 2 x the rate: no gain there; the gain is in LDS bytes and in the
-conversion instructions it removes), and it needs the 8-bit transposing LDS read for V."""
+What it shows: one pass is far inside the bars on the benchmark's inputs, but breaks the LSE bar
+once scores are an order of magnitude larger or the attention is concentrated on a few rows; two
+passes restore it.  So the fp8 contraction has to be the two-term form (2 x the QK matrix work at
+2 x the rate: no gain there; the gain is in LDS bytes and in the conversion instructions it
+removes).  The kernel built on this (flagtree_amd/csrc/smla_mfma_few_f8.hip) goes one step further
+than the variants above: with a POWER-OF-TWO block scale the two e4m3 terms hold a bf16 value
+exactly (last test), so its scores carry no quantisation error of Q at all."""
 import numpy as np
 import pytest
 
@@ -118,3 +120,25 @@ def test_one_pass_breaks_the_lse_bar_on_peaked_attention_and_two_passes_restore_
     res = run(*make(np.random.default_rng(6), 0.3, peaked=True), SM)
     assert res["q_e4m3"][1] > LSE_BAR, res
     assert all(_within(res, v) for v in ("q_split", "q_split+p_e4m3", "q_split+p_split")), res
+
+
+def test_two_e4m3_terms_with_a_power_of_two_scale_hold_a_bf16_value_exactly():
+    """q is bf16: 8 significant bits.  Divided by the power of two that puts the block's largest
+    magnitude into [128, 256) it keeps them; e4m3 takes the top 4 (round to nearest even) and the
+    remainder has at most 4, so hi + lo is q / s exactly wherever the remainder's last bit is on
+    the e4m3 grid: for every value of magnitude >= 2^-9 of the block's largest.  Below that the
+    error is at most half a subnormal step, 2^-10, against a largest value of at least 128."""
+    rng = np.random.default_rng(11)
+    for std in (1e-3, 0.1, 1.0, 40.0):
+        q = oracle.bf16_round((rng.standard_normal((64, 128)) * std * np.exp(rng.standard_normal((64, 128)))).astype(np.float32))
+        am = np.abs(q).max(axis=1, keepdims=True)
+        e = np.floor(np.log2(am))
+        s = (2.0 ** (e - 7)).astype(np.float32)
+        x = q / s
+        assert (np.abs(x) < 256).all() and (np.abs(x).max(axis=1) >= 128).all()
+        hi = e4m3_q(x)
+        lo = e4m3_q(x - hi)
+        err = np.abs((hi + lo).astype(np.float64) - x.astype(np.float64))
+        big = np.abs(x) >= 0.5
+        assert (err[big] == 0).all()
+        assert err.max() <= 2.0 ** -10
