@@ -51,6 +51,8 @@ def parse():
     ap.add_argument("--fp8-mfma", action="store_true",
                     help="decode_fp8 on the kernel that contracts the records' e4m3 codes with fp8 MFMAs (sets "
                          "FLAGTREE_SMLA_FP8_MFMA=1; opt-in until measured)")
+    ap.add_argument("--topk-one-workgroup", action="store_true",
+                    help="topk_* workloads: one workgroup per row even where the rows would be cut into parts")
     ap.add_argument("--token-bands", action="store_true",
                     help="each XCD takes a contiguous band of tokens instead of every eighth one (sets "
                          "FLAGTREE_SMLA_TOKEN_BANDS=1; for prefill_causal_bf16; opt-in until measured)")
@@ -492,14 +494,18 @@ def bench_topk(a, torch, ft, dev):
     g = torch.Generator(device=dev).manual_seed(78)
     sets = [torch.randn((rows, n), generator=g, device=dev) for _ in range(4)]
     nbytes = rows * n * 4 + rows * k * 4                 # every score read once, every index written once
+    # few long rows are cut into parts (two launches on the stream: the parts' selections, then the
+    # rows'); the scratch for the candidates is allocated once, outside the timed loop
+    need = ft.topk_workspace_bytes(rows, n, k)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev) if need and not a.topk_one_workgroup else False
     for i in range(a.warmup):
-        ft.topk_indices(sets[i % 4], k)
+        ft.topk_indices(sets[i % 4], k, workspace=ws)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for i in range(a.steps):
-        ft.topk_indices(sets[i % 4], k)
+        ft.topk_indices(sets[i % 4], k, workspace=ws)
     e1.record()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / a.steps
@@ -509,10 +515,12 @@ def bench_topk(a, torch, ft, dev):
         "metric": "top-k index producer GB/s", "value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": a.workload, "rows": rows, "cols": n, "k": k, "bytes_per_step": nbytes},
+        "config": {"workload": a.workload, "rows": rows, "cols": n, "k": k, "bytes_per_step": nbytes,
+                   "rows_cut_into_parts": ws is not False},
         "roofline": {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
-                     "traffic": measured_traffic(a.workload), "traffic_source": TRAFFIC_NOTE,
-                     "kernel": "topk_resident_kernel", "kernel_ms": kern_ms}}
+                     "traffic": None if ws is not False else measured_traffic(a.workload), "traffic_source": TRAFFIC_NOTE,
+                     "kernel": "topk_part_kernel + topk_merge_kernel" if ws is not False else "topk_resident_kernel",
+                     "kernel_ms": kern_ms}}
     if not a.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         import oracle

@@ -103,7 +103,7 @@ const char* smla_strerror(int status) {
   return "unknown status";
 }
 
-int smla_abi_version(void) { return 3; }
+int smla_abi_version(void) { return 4; }
 
 int smla_merge_in_launch(void) { return merge_in_launch_ok() ? 1 : 0; }
 
@@ -327,12 +327,19 @@ int smla_kv_write(int kv_format, const void* latent, const int64_t* slot_mapping
   return SMLA_EINVAL_SHAPE;
 }
 
+size_t smla_topk_workspace_bytes(int32_t n_rows, int32_t n_cols, int32_t k) {
+  if (n_rows <= 0 || n_cols <= 0 || k <= 0) return 0;
+  return topk_workspace_bytes(n_rows, n_cols, k, device_cus());
+}
+
 int smla_topk_indices(const float* scores, const int32_t* context_lens, int32_t* indices_out,
-                      int32_t n_rows, int32_t n_cols, int64_t row_stride, int32_t k, void* stream) {
+                      int32_t n_rows, int32_t n_cols, int64_t row_stride, int32_t k, void* workspace,
+                      size_t workspace_bytes, void* stream) {
   if (!scores || !indices_out) return SMLA_EINVAL_NULLPTR;
   if (n_rows < 0 || n_cols <= 0 || k <= 0 || row_stride < n_cols) return SMLA_EINVAL_SHAPE;
-  return launch_topk_indices(scores, context_lens, indices_out, n_rows, n_cols, row_stride, k,
-                             static_cast<hipStream_t>(stream));
+  if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return SMLA_EINVAL_ALIGN;
+  return launch_topk_indices(scores, context_lens, indices_out, n_rows, n_cols, row_stride, k, workspace,
+                             workspace_bytes, device_cus(), static_cast<hipStream_t>(stream));
 }
 
 int smla_gemm_rs_local(const void* x, const void* w, const float* partial, void* out, int32_t m,

@@ -242,7 +242,9 @@ int launch_quantize(const void* src, const int64_t* slot, void* records, int64_t
                     int64_t record_rows, hipStream_t s);
 int launch_kv_copy(const void* src, const int64_t* slot, void* pool, int64_t n_rows, int64_t pool_rows, hipStream_t s);
 int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_t* out, int n_rows,
-                        int n_cols, long long row_stride, int k, hipStream_t s);
+                        int n_cols, long long row_stride, int k, void* workspace, size_t workspace_bytes, int n_cu,
+                        hipStream_t s);
+size_t topk_workspace_bytes(int n_rows, int n_cols, int k, int n_cu);
 int launch_zero(void* ptr, size_t bytes, hipStream_t s);
 int launch_workspace_init(void* workspace, hipStream_t s);
 int launch_gemm_rs(const void* x, const void* w, const float* partial, void* out, int m, int n,

@@ -13,6 +13,16 @@
 // through all passes (topk_resident_kernel); longer rows are walked from memory in every pass
 // and stay in L2 between them (topk_stream_kernel).
 // Entries at or past the row's context length do not take part; NaN ranks with -inf.
+//
+// Few long rows (fewer rows than half the compute units, given a workspace): a row is cut into
+// parts of equal length, one workgroup each, and every part selects ITS k largest entries by the
+// same rule (topk_part_kernel).  An entry of the row's answer is in its part's answer: if it were
+// not, k entries of the part would rank ahead of it, and so would they in the row.  The parts'
+// answers (key and index of every entry, in index order, parts in index order) are one candidate
+// list per row in the workspace, still in ascending index order, and a second launch selects the
+// row's k largest from it, again by the same rule, reading the indices through the list
+// (topk_merge_kernel).  Ties at the k-th value go to the candidate that comes first, which is the
+// one of lower index: the answer is the same list, entry for entry, as one workgroup gives.
 #include "smla_common.h"
 
 namespace smla {
@@ -144,12 +154,26 @@ __device__ __forceinline__ void turn_round(const float4 (&q)[4], int lane, float
   __builtin_amdgcn_wave_barrier();
 }
 
-// R = rounds a wavefront can hold (16 R keys a lane); a row of up to 1024 R WAVES entries.
-template <int WAVES, int R>
-__global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* __restrict__ scores,
-                                                                  const int32_t* __restrict__ context_lens,
-                                                                  int32_t* __restrict__ out, int n_cols,
-                                                                  long long row_stride, int k) {
+// What a selection reads and writes:
+//   kWhole  scores of a whole row -> the row's answer (indices)
+//   kPart   scores of one part of a row -> the part's answer as candidates (key and index of each)
+//   kMerge  a row's candidate keys (entry j of `x` is a key's bit pattern, never 0) -> the row's
+//           answer, entry j standing for index cand_idx[j]
+enum { kWhole = 0, kPart = 1, kMerge = 2 };
+template <int MODE>
+__device__ __forceinline__ uint32_t key_of(float x) {
+  if constexpr (MODE == kMerge) return __float_as_uint(x);
+  else return score_key(x);
+}
+
+// R = rounds a wavefront can hold (16 R keys a lane); `n` entries at x (up to 1024 R WAVES), the
+// `want` largest wanted.  Entry i stands for index index0 + i (kWhole, kPart) or cand_idx[i]
+// (kMerge).  The answer goes to o[0 .. want) (kWhole, kMerge) or, key and index, to cand_key_out /
+// cand_idx_out[0 .. want) (kPart).
+template <int WAVES, int R, int MODE>
+__device__ __forceinline__ void resident_select(const float* __restrict__ x, int n, int want, int index0,
+                                                const int32_t* __restrict__ cand_idx, int32_t* __restrict__ o,
+                                                uint32_t* __restrict__ cand_key_out, int32_t* __restrict__ cand_idx_out) {
   constexpr int kThreads = 64 * WAVES;
   // copies of every histogram bin, picked by lane % kCopies: score exponents are heavily skewed,
   // and lanes adding to one LDS word serialise.  A workgroup of 16 wavefronts has the LDS for one
@@ -169,12 +193,6 @@ __global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* 
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int row = blockIdx.x;
-  const float* x = scores + (size_t)row * row_stride;
-  int32_t* o = out + (size_t)row * k;
-  const int n = context_lens ? max(0, min(context_lens[row], n_cols)) : n_cols;
-  const int want = min(k, n);                   // entries to select
-  for (int j = want + tid; j < k; j += kThreads) o[j] = -1;
   if (want == 0) return;
   const bool vec = ((uintptr_t)x & 15) == 0;
 
@@ -196,10 +214,10 @@ __global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* 
       const int i0 = seg0 + kRound * r + 16 * lane;
       if (seg0 + kRound * (r + 1) <= seg1) {    // wave-uniform: a full round needs no liveness test
 #pragma unroll
-        for (int j = 0; j < 16; ++j) key[r][j] = score_key(v[j]);
+        for (int j = 0; j < 16; ++j) key[r][j] = key_of<MODE>(v[j]);
       } else {
 #pragma unroll
-        for (int j = 0; j < 16; ++j) key[r][j] = i0 + j < seg1 ? score_key(v[j]) : 0u;
+        for (int j = 0; j < 16; ++j) key[r][j] = i0 + j < seg1 ? key_of<MODE>(v[j]) : 0u;
       }
     } else {
 #pragma unroll
@@ -402,11 +420,18 @@ __global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* 
   int above_before = 0, equal_before = 0;
   for (int w = 0; w < wave; ++w) { above_before += (int)s_tot[2 * w]; equal_before += (int)s_tot[2 * w + 1]; }
 
-  // ---- 3. write the selected indices out in ascending order: (round, lane, entry) within the
+  // ---- 3. write the selected entries out in ascending order: (round, lane, entry) within the
   // wavefront.  Neighbouring lanes' outputs lie a few entries apart, so when the list fits the LDS
-  // it is put together there and copied out in whole lines.
+  // it is put together there (as positions in x) and copied out in whole lines.  What a position
+  // stands for is looked up on the way out: the index itself, the candidate's index, or (a part's
+  // answer) index and key, the key recomputed from the score, which is in L2.
   int32_t* s_list = reinterpret_cast<int32_t*>(s_raw);
   const bool staged = want <= kRawWords;
+  auto emit = [&](int at, int pos) {
+    if constexpr (MODE == kWhole) o[at] = index0 + pos;
+    else if constexpr (MODE == kMerge) o[at] = cand_idx[pos];
+    else { cand_idx_out[at] = index0 + pos; cand_key_out[at] = score_key(x[pos]); }
+  };
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (r < n_rounds) {
@@ -429,7 +454,7 @@ __global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* 
       while (sel != 0u) {
         const int j = __builtin_ctz(sel);
         if (staged) s_list[at] = i0 + j;
-        else o[at] = i0 + j;
+        else emit(at, i0 + j);
         ++at;
         sel &= sel - 1u;
       }
@@ -439,8 +464,61 @@ __global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* 
   }
   if (staged) {
     __syncthreads();
-    for (int j = tid; j < want; j += kThreads) o[j] = s_list[j];
+    for (int j = tid; j < want; j += kThreads) emit(j, s_list[j]);
   }
+}
+
+template <int WAVES, int R>
+__global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* __restrict__ scores,
+                                                                  const int32_t* __restrict__ context_lens,
+                                                                  int32_t* __restrict__ out, int n_cols,
+                                                                  long long row_stride, int k) {
+  const int row = blockIdx.x;
+  const int n = context_lens ? max(0, min(context_lens[row], n_cols)) : n_cols;
+  const int want = min(k, n);                   // entries to select
+  int32_t* o = out + (size_t)row * k;
+  for (int j = want + (int)threadIdx.x; j < k; j += 64 * WAVES) o[j] = -1;
+  resident_select<WAVES, R, kWhole>(scores + (size_t)row * row_stride, n, want, 0, nullptr, o, nullptr, nullptr);
+}
+
+// ---- a row cut into parts ----------------------------------------------------------------------
+// Part p of a row holds entries [p part_len, (p + 1) part_len) below the row's context length and
+// answers with min(k, its length) candidates; the row's candidates lie back to back from
+// (row * n_parts) * k on, part after part, so that entry j of the list is a position in index order.
+__device__ __forceinline__ int part_answers(int n, int part_len, int k, int p) {
+  return min(k, max(0, min(n - p * part_len, part_len)));
+}
+
+template <int WAVES, int R>
+__global__ __launch_bounds__(64 * WAVES) void topk_part_kernel(const float* __restrict__ scores,
+                                                              const int32_t* __restrict__ context_lens,
+                                                              uint32_t* __restrict__ cand_key, int32_t* __restrict__ cand_idx,
+                                                              int n_cols, long long row_stride, int k, int n_parts, int part_len) {
+  const int row = blockIdx.x / n_parts, part = blockIdx.x % n_parts;
+  const int n = context_lens ? max(0, min(context_lens[row], n_cols)) : n_cols;
+  int before = 0;
+  for (int p = 0; p < part; ++p) before += part_answers(n, part_len, k, p);
+  const int want = part_answers(n, part_len, k, part);
+  const size_t base = (size_t)row * n_parts * k + before;
+  const int first = part * part_len;
+  resident_select<WAVES, R, kPart>(scores + (size_t)row * row_stride + first, max(0, min(n - first, part_len)), want, first, nullptr,
+                                   nullptr, cand_key + base, cand_idx + base);
+}
+
+template <int WAVES, int R>
+__global__ __launch_bounds__(64 * WAVES) void topk_merge_kernel(const uint32_t* __restrict__ cand_key,
+                                                               const int32_t* __restrict__ cand_idx,
+                                                               const int32_t* __restrict__ context_lens,
+                                                               int32_t* __restrict__ out, int n_cols, int k, int n_parts, int part_len) {
+  const int row = blockIdx.x;
+  const int n = context_lens ? max(0, min(context_lens[row], n_cols)) : n_cols;
+  int n_cand = 0;
+  for (int p = 0; p < n_parts; ++p) n_cand += part_answers(n, part_len, k, p);
+  const int want = min(k, n);                   // (== min(k, n_cand): every part answers with all it has, up to k)
+  int32_t* o = out + (size_t)row * k;
+  for (int j = want + (int)threadIdx.x; j < k; j += 64 * WAVES) o[j] = -1;
+  const size_t base = (size_t)row * n_parts * k;
+  resident_select<WAVES, R, kMerge>(reinterpret_cast<const float*>(cand_key + base), n_cand, want, 0, cand_idx + base, o, nullptr, nullptr);
 }
 
 // Rows of any length: every pass walks the row in memory.
@@ -578,9 +656,57 @@ __global__ __launch_bounds__(64 * WAVES) void topk_stream_kernel(const float* __
 
 }  // namespace
 
+// How many parts a row is cut into (1: not at all).  Cutting pays when the rows alone leave most
+// compute units idle and a part is still long enough to be worth a workgroup; a part must fit the
+// register-resident selection (65 536 entries) and so must the candidates of a row (n_parts * k).
+int topk_parts(int n_rows, int n_cols, int k, int n_cu, int* part_len_out) {
+  int parts = 1;
+  if (n_rows > 0 && 2 * n_rows <= n_cu && n_cols >= 8192) {
+    parts = n_cu / n_rows;
+    if (parts > 8) parts = 8;
+    while (parts > 1 && (n_cols + parts - 1) / parts < 4096) --parts;
+    while (parts > 1 && (long long)parts * k > 65536) --parts;
+  }
+  int part_len = ((n_cols + parts - 1) / parts + 1023) & ~1023;
+  if (parts > 1 && part_len > 65536) { parts = 1; part_len = n_cols; }
+  if (parts > 1) parts = (n_cols + part_len - 1) / part_len;      // (rounding the length up may leave the last part empty)
+  if (part_len_out) *part_len_out = part_len;
+  return parts;
+}
+
+size_t topk_workspace_bytes(int n_rows, int n_cols, int k, int n_cu) {
+  const int parts = topk_parts(n_rows, n_cols, k, n_cu, nullptr);
+  return parts > 1 ? (size_t)n_rows * parts * k * 8 : 0;
+}
+
 int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_t* out, int n_rows,
-                        int n_cols, long long row_stride, int k, hipStream_t s) {
+                        int n_cols, long long row_stride, int k, void* workspace, size_t workspace_bytes, int n_cu,
+                        hipStream_t s) {
   if (n_rows == 0) return SMLA_OK;
+  int part_len = n_cols;
+  const int parts = topk_parts(n_rows, n_cols, k, n_cu, &part_len);
+  if (parts > 1 && workspace != nullptr && workspace_bytes >= (size_t)n_rows * parts * k * 8) {
+    uint32_t* cand_key = static_cast<uint32_t*>(workspace);
+    int32_t* cand_idx = reinterpret_cast<int32_t*>(cand_key + (size_t)n_rows * parts * k);
+    const dim3 grid1((unsigned)(n_rows * parts));
+    if (part_len <= 4096)
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_part_kernel<4, 1>), grid1, dim3(256), 0, s, scores, context_lens, cand_key, cand_idx, n_cols, row_stride, k, parts, part_len);
+    else if (part_len <= 16384)
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_part_kernel<16, 1>), grid1, dim3(1024), 0, s, scores, context_lens, cand_key, cand_idx, n_cols, row_stride, k, parts, part_len);
+    else
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_part_kernel<16, 4>), grid1, dim3(1024), 0, s, scores, context_lens, cand_key, cand_idx, n_cols, row_stride, k, parts, part_len);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_status(e);
+    const dim3 grid2((unsigned)n_rows);
+    const long long n_cand = (long long)parts * k;
+    if (n_cand <= 4096)
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<4, 1>), grid2, dim3(256), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len);
+    else if (n_cand <= 16384)
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<16, 1>), grid2, dim3(1024), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len);
+    else
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<16, 4>), grid2, dim3(1024), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len);
+    return hip_status(hipGetLastError());
+  }
   const dim3 grid((unsigned)n_rows);
   // Rows of up to 65 536 entries are held in registers, 16 or 64 entries a lane.  With many rows a
   // CU works on several at once and what counts is instructions per row: few wavefronts (the

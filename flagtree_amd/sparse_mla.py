@@ -353,11 +353,15 @@ def reshape_and_cache(latent, kv_cache, slot_mapping, kv_format="bf16"):
     _lib.check(rc, "smla_kv_write")
 
 
-def topk_indices(scores, k, context_lens=None):
+def topk_indices(scores, k, context_lens=None, workspace=None):
     """Top-k index producer: int32 [..., k] indices of the k largest entries of each row of ``scores``
     (f32 [..., N]) among its first ``context_lens[row]`` entries (default N), ascending, -1 padded.
     Ties at the k-th value go to the lower index.  The reference only has ``topk`` as a language
-    primitive returning values (/root/reference/third_party/metax/python/triton/language/standard.py:443)."""
+    primitive returning values (/root/reference/third_party/metax/python/triton/language/standard.py:443).
+    Few long rows are cut into parts, one workgroup each, through a scratch buffer: ``workspace``
+    (a uint8 device tensor of ``topk_workspace_bytes`` bytes, e.g. kept by a serving loop), or one
+    allocated here for the call; ``workspace=False`` keeps one workgroup per row.  Same result
+    every way."""
     if not _lib.on_device(scores):
         raise ValueError("topk_indices needs device tensors (there is no CPU path)")
     if scores.dtype != torch.float32:
@@ -375,10 +379,26 @@ def topk_indices(scores, k, context_lens=None):
         if cl.shape[0] != rows or not _lib.on_device(cl):
             raise ValueError("context_lens needs one device entry per row")
     out = torch.empty((rows, k), dtype=torch.int32, device=scores.device)
-    rc = _lib.load().smla_topk_indices(s2.data_ptr(), cl.data_ptr() if cl is not None else None, out.data_ptr(),
-                                       rows, n, s2.stride(0) if rows > 1 else n, k, _stream(s2))
+    lib = _lib.load()
+    need = lib.smla_topk_workspace_bytes(rows, n, k)
+    if workspace is False:
+        workspace = None
+    elif workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=scores.device)
+    elif workspace is not None:
+        if workspace.dtype != torch.uint8 or not workspace.is_contiguous() or not _lib.on_device(workspace):
+            raise ValueError("workspace must be a contiguous uint8 device tensor")
+    rc = lib.smla_topk_indices(s2.data_ptr(), cl.data_ptr() if cl is not None else None, out.data_ptr(),
+                               rows, n, s2.stride(0) if rows > 1 else n, k,
+                               workspace.data_ptr() if workspace is not None else None,
+                               workspace.numel() if workspace is not None else 0, _stream(s2))
     _lib.check(rc, "smla_topk_indices")
     return out.reshape(*lead, k)
+
+
+def topk_workspace_bytes(n_rows, n_cols, k):
+    """Bytes of scratch with which ``topk_indices`` cuts rows of this shape into parts (0: it would not)."""
+    return _lib.load().smla_topk_workspace_bytes(n_rows, n_cols, k)
 
 
 def decode_attention_fwd(q, k_buffer, v_buffer, o, req_to_token, b_seq_len, attn_logits=None, num_kv_splits=None,

@@ -238,9 +238,21 @@ int smla_kv_write(int kv_format, const void* latent, const int64_t* slot_mapping
  * The reference has the selection only as a language-level primitive that returns the k largest
  * values (/root/reference/third_party/metax/python/triton/language/standard.py:443-444, bitonic
  * top-k :399-435); returning indices, their order and the tie rule are this library's decisions.
+ *   workspace  optional device scratch (4-byte aligned) of at least smla_topk_workspace_bytes() bytes, or
+ *   NULL.  With few long rows (fewer rows than half the device's compute units) and a workspace,
+ *   a row is cut into parts that select their own k largest entries, one workgroup each, and a
+ *   second launch on the same stream selects the row's answer from the parts' (same list, entry
+ *   for entry, as without a workspace).  Without one, or when the shape does not call for it,
+ *   one workgroup takes a row.  The workspace needs no initialisation and carries nothing from
+ *   call to call.
  */
 int smla_topk_indices(const float* scores, const int32_t* context_lens, int32_t* indices_out,
-                      int32_t n_rows, int32_t n_cols, int64_t row_stride, int32_t k, void* stream);
+                      int32_t n_rows, int32_t n_cols, int64_t row_stride, int32_t k, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+/* Bytes of workspace with which smla_topk_indices cuts rows of this shape into parts on the current
+ * device; 0 when it would not (many rows, short rows).  No counterpart in the reference. */
+size_t smla_topk_workspace_bytes(int32_t n_rows, int32_t n_cols, int32_t k);
 
 /*
  * Local GEMM of GEMM + reduce-scatter with chunked-output epilogue:

@@ -132,7 +132,10 @@ def topk_case(seed, rng, g, end):
     out = G(torch.full((rows, k), -9, dtype=torch.int32), end).tensor
     print(f"seed {seed} topk rows={rows} n={n} k={k} stride={stride} lens={lens is not None}", flush=True)
     random_schedule(rng)
-    rc = lib.smla_topk_indices(sc.data_ptr(), lens.data_ptr() if lens is not None else None, out.data_ptr(), rows, n, stride, k, None)
+    need = lib.smla_topk_workspace_bytes(rows, n, k)
+    ws = G(torch.full((need,), 0x5A, dtype=torch.uint8), end).tensor if need and rng.random() < 0.7 else None      # rows cut into parts
+    rc = lib.smla_topk_indices(sc.data_ptr(), lens.data_ptr() if lens is not None else None, out.data_ptr(), rows, n, stride, k,
+                               ws.data_ptr() if ws is not None else None, need if ws is not None else 0, None)
     assert rc == 0, rc
     want = oracle.topk_indices(to_np(buf)[:, :n], k, to_np(lens_t) if lens is not None else None)
     assert np.array_equal(to_np(out), want)

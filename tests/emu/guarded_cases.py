@@ -107,7 +107,13 @@ def _topk(G):
         scores = G(torch.randn((rows, n), generator=g))
         lens = G(torch.randint(1, n + 1, (rows,), generator=g, dtype=torch.int32))
         out = G(torch.zeros((rows, k), dtype=torch.int32))
-        assert harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), rows, n, n, k, None) == 0
+        assert harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), rows, n, n, k, None, 0, None) == 0
+        need = harness.lib().smla_topk_workspace_bytes(rows, n, k)      # rows cut into parts: the candidate lists in a guarded workspace
+        if need:
+            ws = G(torch.zeros(need, dtype=torch.uint8))
+            out2 = G(torch.zeros((rows, k), dtype=torch.int32))
+            assert harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out2.data_ptr(), rows, n, n, k, ws.data_ptr(), need, None) == 0
+            assert torch.equal(out, out2)
 
 
 def _gemm(G):

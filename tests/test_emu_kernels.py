@@ -757,7 +757,7 @@ def test_topk_indices_exact(rows, n, k):
     for skew in (0, 1, 2):
         harness.configure(wave_skew_seed=skew)
         out = torch.full((rows, k), -9, dtype=torch.int32)
-        rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), rows, n, n, k, None)
+        rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), rows, n, n, k, None, 0, None)
         assert rc == 0
         assert np.array_equal(to_np(out), want), skew
     harness.configure()
@@ -777,10 +777,80 @@ def test_topk_indices_with_tied_values_in_long_rows(n, length, k):
     for skew in (0, 1):
         harness.configure(wave_skew_seed=skew)
         out = torch.full((2, k), -9, dtype=torch.int32)
-        rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), 2, n, n, k, None)
+        rc = harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), 2, n, n, k, None, 0, None)
         assert rc == 0
         assert np.array_equal(to_np(out), want), skew
     harness.configure()
+
+
+@pytest.mark.parametrize("rows,n,k", [(1, 20000, 300), (2, 65536, 2048), (3, 8192, 64), (1, 70001, 2048), (2, 300000, 128), (1, 9000, 9000)])
+def test_topk_rows_cut_into_parts_give_the_same_list(rows, n, k):
+    """Few long rows with a workspace: every part of a row selects its own k largest, a second
+    launch selects the row's from the parts' candidates.  Exact against the oracle and entry for
+    entry what one workgroup per row gives: ties (quantised scores) at the k-th value, also across
+    part boundaries, NaN, -inf, context lengths that end inside the first part or leave parts empty."""
+    lib = harness.lib()
+    need = lib.smla_topk_workspace_bytes(rows, n, k)
+    assert need > 0
+    g = torch.Generator().manual_seed(rows * 1000 + k)
+    for case in range(4):
+        scores = torch.randn((rows, n), generator=g)
+        if case >= 1:
+            scores = (scores * 2).round() / 2                           # heavy ties
+        if case == 2:
+            scores[0, : n // 2] = float("-inf")
+            scores[-1, n // 3] = float("nan")
+        lens = torch.tensor([n, max(1, n // 5), 3][:rows], dtype=torch.int32)
+        if case == 3:
+            lens = torch.tensor([n - 1, 4097, 0][:rows], dtype=torch.int32)
+        want = oracle.topk_indices(to_np(scores), k, to_np(lens))
+        for skew in (0, 3):
+            harness.configure(wave_skew_seed=skew, concurrent_blocks=4 if skew else 0, concurrent_seed=5)
+            ws = torch.full((need,), 0x5A, dtype=torch.uint8)
+            out = torch.full((rows, k), -9, dtype=torch.int32)
+            launches = lib.emu_launch_count()
+            rc = lib.smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out.data_ptr(), rows, n, n, k, ws.data_ptr(), need, None)
+            assert rc == 0 and lib.emu_launch_count() - launches == 2
+            assert np.array_equal(to_np(out), want), (case, skew)
+    harness.configure()
+    # too small a workspace, or none: one workgroup per row, same answer
+    out1 = torch.full((rows, k), -9, dtype=torch.int32)
+    launches = lib.emu_launch_count()
+    assert lib.smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out1.data_ptr(), rows, n, n, k, ws.data_ptr(), need - 1, None) == 0
+    assert lib.emu_launch_count() - launches == 1 and np.array_equal(to_np(out1), want)
+
+
+def test_topk_tie_run_across_a_part_boundary():
+    """All entries equal around the boundary between two parts: the k-th place falls inside the run,
+    and the entries taken are the ones of lowest index, whichever part they lie in."""
+    lib = harness.lib()
+    n, k = 16384, 5000
+    need = lib.smla_topk_workspace_bytes(1, n, k)
+    assert need > 0
+    scores = torch.zeros((1, n))
+    scores[0, 100:3000] = 1.0                                          # 2900 entries above the run, all in the first part
+    scores[0, 12000:12100] = 2.0                                       # 100 more in a later part
+    want = oracle.topk_indices(to_np(scores), k, None)
+    assert (want[0] >= 0).all() and want[0].max() < 12100
+    ws = torch.zeros(need, dtype=torch.uint8)
+    out = torch.full((1, k), -9, dtype=torch.int32)
+    assert lib.smla_topk_indices(scores.data_ptr(), None, out.data_ptr(), 1, n, n, k, ws.data_ptr(), need, None) == 0
+    assert np.array_equal(to_np(out), want)
+
+
+def test_topk_part_planning():
+    lib = harness.lib()
+    try:
+        lib.emu_set_cu_count(256)
+        assert lib.smla_topk_workspace_bytes(64, 65536, 2048) == 64 * 4 * 2048 * 8        # the decode shape: four parts a row
+        assert lib.smla_topk_workspace_bytes(4096, 4096, 2048) == 0                       # many short rows: one workgroup a row
+        assert lib.smla_topk_workspace_bytes(200, 65536, 2048) == 0                       # rows alone fill most of the device
+        assert lib.smla_topk_workspace_bytes(1, 1 << 20, 2048) == 0                       # parts would not fit the registers
+        assert lib.smla_topk_workspace_bytes(1, 400000, 2048) == 8 * 2048 * 8             # 8 parts of 50 176 entries
+        assert lib.smla_topk_workspace_bytes(1, 33000, 2048) == 7 * 2048 * 8              # 8 parts of 5120 would leave the last one empty: 7
+        assert lib.smla_topk_workspace_bytes(8, 65536, 20000) == 8 * 3 * 20000 * 8        # candidates of a row must fit too
+    finally:
+        lib.emu_set_cu_count(harness.EMU_CUS)
 
 
 @pytest.mark.parametrize("m,n,k,chunks", [(256, 256, 128, 2), (128, 512, 192, 1), (384, 256, 64, 3), (512, 256, 128, 4),

@@ -256,6 +256,8 @@ def test_reshape_and_cache_both_formats(dev):
 @pytest.mark.parametrize("n,k,quant", [(1, 1, 0), (37, 64, 0), (1024, 1024, 0), (1500, 256, 0), (4096, 2048, 8),
                                        (65536, 2048, 0), (65536, 2048, 64), (10000, 2048, 2)])
 def test_topk_indices_exact(dev, n, k, quant):
+    """(The rows of 10 000 and 65 536 entries are cut into parts when the wrapper may allocate a
+    workspace; both ways must give the oracle's list.)"""
     import flagtree_amd as ft
     g = np.random.default_rng(1000 + n + k)
     x = g.standard_normal((5, n)).astype(np.float32)
@@ -268,6 +270,8 @@ def test_topk_indices_exact(dev, n, k, quant):
     assert np.array_equal(to_np(got), oracle.topk_indices(x, k, lens))
     got2 = ft.topk_indices(torch.from_numpy(x).to(dev), k)
     assert np.array_equal(to_np(got2), oracle.topk_indices(x, k))
+    got3 = ft.topk_indices(torch.from_numpy(x).to(dev), k, torch.from_numpy(lens).to(dev), workspace=False)
+    assert np.array_equal(to_np(got3), oracle.topk_indices(x, k, lens))
 
 
 @pytest.mark.parametrize("rows,n,k,quant", [(1100, 4096, 300, 0),      # many short rows
@@ -287,6 +291,9 @@ def test_topk_indices_shapes(dev, rows, n, k, quant):
     lens[:3] = [n, 1, 0][:min(3, rows)]
     got = ft.topk_indices(torch.from_numpy(x).to(dev), k, torch.from_numpy(lens).to(dev))
     assert np.array_equal(to_np(got), oracle.topk_indices(x, k, lens))
+    if ft.topk_workspace_bytes(rows, n, k):                        # cut into parts above: also one workgroup per row
+        got = ft.topk_indices(torch.from_numpy(x).to(dev), k, torch.from_numpy(lens).to(dev), workspace=False)
+        assert np.array_equal(to_np(got), oracle.topk_indices(x, k, lens))
 
 
 @pytest.mark.parametrize("n", [1000, 4099, 20000])
@@ -317,8 +324,10 @@ def test_topk_indices_degenerate_rows(dev, n, k):
     rows.append(tied)
     x = np.stack(rows).astype(np.float32)
     got = ft.topk_indices(torch.from_numpy(x).to(dev), k)
+    got1 = ft.topk_indices(torch.from_numpy(x).to(dev), k, workspace=False)
     with np.errstate(all="ignore"):
         assert np.array_equal(to_np(got), oracle.topk_indices(x, k))
+        assert np.array_equal(to_np(got1), oracle.topk_indices(x, k))
 
 
 def test_topk_feeds_sparse_mla(dev):

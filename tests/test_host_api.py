@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
         assert hasattr(lib, n), f"{n} declared in include/flagtree_smla.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.smla_abi_version() == 3
+    assert lib.smla_abi_version() == 4
 
 
 def test_status_texts(lib):
@@ -82,10 +82,10 @@ def test_validation_codes_without_a_device(lib):
     assert lib.smla_kv_write(0, p16 + 4, None, p16, 4, 64, None) == -3
     assert lib.smla_kv_write(7, p16, None, p16, 4, 64, None) == -2                           # unknown cache format
     assert lib.smla_kv_quantize_fp8(p16, None, p16, 4, 0, None) == -2 and lib.smla_kv_quantize_fp8(p16 + 8, None, p16, 4, 8, None) == -3
-    assert lib.smla_topk_indices(None, None, p16, 1, 64, 64, 8, None) == -1 and lib.smla_topk_indices(p16, None, None, 1, 64, 64, 8, None) == -1
-    assert lib.smla_topk_indices(p16, None, p16, 1, 0, 64, 8, None) == -2 and lib.smla_topk_indices(p16, None, p16, 1, 64, 64, 0, None) == -2
-    assert lib.smla_topk_indices(p16, None, p16, -1, 64, 64, 8, None) == -2
-    assert lib.smla_topk_indices(p16, None, p16, 1, 64, 32, 8, None) == -2                   # row stride shorter than a row
+    assert lib.smla_topk_indices(None, None, p16, 1, 64, 64, 8, None, 0, None) == -1 and lib.smla_topk_indices(p16, None, None, 1, 64, 64, 8, None, 0, None) == -1
+    assert lib.smla_topk_indices(p16, None, p16, 1, 0, 64, 8, None, 0, None) == -2 and lib.smla_topk_indices(p16, None, p16, 1, 64, 64, 0, None, 0, None) == -2
+    assert lib.smla_topk_indices(p16, None, p16, -1, 64, 64, 8, None, 0, None) == -2
+    assert lib.smla_topk_indices(p16, None, p16, 1, 64, 32, 8, None, 0, None) == -2                   # row stride shorter than a row
 
     def dense(**kw):
         a = dict(ok, **kw)

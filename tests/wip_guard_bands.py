@@ -107,7 +107,7 @@ def test_topk_indices_stays_inside_its_buffer(dev, rows, n, k):
     scores = torch.randn((rows, n), generator=g, device=dev)
     lens = torch.randint(0, n + 1, (rows,), generator=g, device=dev, dtype=torch.int32)
     out_b = Banded(rows * k * 4, dev)
-    rc = _lib.load().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out_b.ptr(), rows, n, n, k, _stream(dev))
+    rc = _lib.load().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out_b.ptr(), rows, n, n, k, None, 0, _stream(dev))
     _lib.check(rc, "smla_topk_indices")
     torch.cuda.synchronize()
     ref = ft.topk_indices(scores, k, context_lens=lens)
