@@ -37,6 +37,7 @@ SIGNATURES = {
     "smla_kv_quantize_fp8": (_c.c_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "smla_kv_write": (_c.c_int, [_c.c_int, _vp, _vp, _vp, _i64, _i64, _vp]),
     "smla_topk_indices": (_c.c_int, [_vp, _vp, _vp, _c.c_int32, _c.c_int32, _i64, _c.c_int32, _vp, _sz, _vp]),
+    "smla_topk_rows": (_c.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i32, _i32, _i64, _vp, _sz, _vp]),
     "smla_topk_workspace_bytes": (_sz, [_i32, _i32, _i32]),
     "smla_gemm_rs_local": (_c.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, _vp]),
 }

@@ -338,7 +338,21 @@ int smla_topk_indices(const float* scores, const int32_t* context_lens, int32_t*
   if (!scores || !indices_out) return SMLA_EINVAL_NULLPTR;
   if (n_rows < 0 || n_cols <= 0 || k <= 0 || row_stride < n_cols) return SMLA_EINVAL_SHAPE;
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return SMLA_EINVAL_ALIGN;
-  return launch_topk_indices(scores, context_lens, indices_out, n_rows, n_cols, row_stride, k, workspace,
+  return launch_topk_indices(scores, context_lens, indices_out, n_rows, n_cols, row_stride, k, TopkPaging{nullptr, 0, 1, 1, 0},
+                             workspace, workspace_bytes, device_cus(), static_cast<hipStream_t>(stream));
+}
+
+int smla_topk_rows(const float* scores, const int32_t* context_lens, const int32_t* block_table, int32_t* rows_out,
+                   int32_t n_rows, int32_t n_cols, int64_t row_stride, int32_t k, int32_t rows_per_seq,
+                   int32_t page_size, int32_t block_table_stride, int64_t kv_rows, void* workspace,
+                   size_t workspace_bytes, void* stream) {
+  if (!scores || !rows_out || !block_table) return SMLA_EINVAL_NULLPTR;
+  if (n_rows < 0 || n_cols <= 0 || k <= 0 || row_stride < n_cols) return SMLA_EINVAL_SHAPE;
+  if (rows_per_seq <= 0 || n_rows % rows_per_seq != 0 || page_size <= 0 || block_table_stride <= 0) return SMLA_EINVAL_SHAPE;
+  if (kv_rows <= 0 || kv_rows > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
+  if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return SMLA_EINVAL_ALIGN;
+  return launch_topk_indices(scores, context_lens, rows_out, n_rows, n_cols, row_stride, k,
+                             TopkPaging{block_table, block_table_stride, page_size, rows_per_seq, kv_rows}, workspace,
                              workspace_bytes, device_cus(), static_cast<hipStream_t>(stream));
 }
 

@@ -72,17 +72,23 @@ __device__ __forceinline__ int32_t list_entry(const Params& p, int t, int seq, i
   return j < p.seq_lens[seq] ? j : -1;
 }
 
-// Logical top-k entry -> physical row, -1 when masked.  Integer-only.  `bt_row` is the sequence's
-// page-table row (any address space the caller has it in); only used when the cache is paged.
-__device__ __forceinline__ int32_t translate_index(const Params& p, int32_t idx, const int32_t* bt_row) {
+// Logical position -> physical row of a paged cache, -1 when masked (negative, past the table,
+// a negative page number, or a row past the pool).  Integer-only.  `bt_row` is the sequence's
+// page-table row (any address space the caller has it in).
+__device__ __forceinline__ int32_t paged_row(int32_t idx, const int32_t* bt_row, int32_t bt_stride, int32_t page_size, int64_t kv_rows) {
   // (branch-free, the page lookup is unconditional: loads inside branches would be issued one
   // at a time, each waiting for the one before it)
-  const int64_t cap = (int64_t)p.bt_stride * p.page_size;
+  const int64_t cap = (int64_t)bt_stride * page_size;
   const bool in_table = idx >= 0 && idx < cap;
   const int32_t safe = in_table ? idx : 0;
-  const int32_t page = bt_row[safe / p.page_size];
-  const int64_t phys = (int64_t)page * p.page_size + safe % p.page_size;
-  return in_table && page >= 0 && phys < p.kv_rows ? (int32_t)phys : -1;
+  const int32_t page = bt_row[safe / page_size];
+  const int64_t phys = (int64_t)page * page_size + safe % page_size;
+  return in_table && page >= 0 && phys < kv_rows ? (int32_t)phys : -1;
+}
+
+// Logical top-k entry -> physical row, -1 when masked; only used when the cache is paged.
+__device__ __forceinline__ int32_t translate_index(const Params& p, int32_t idx, const int32_t* bt_row) {
+  return paged_row(idx, bt_row, p.bt_stride, p.page_size, p.kv_rows);
 }
 
 __device__ __forceinline__ int32_t translate_unpaged(const Params& p, int seq, int32_t idx) {
@@ -241,9 +247,16 @@ int launch_gather(const Params& p, int row_bytes, int32_t* phys_out, void* rows_
 int launch_quantize(const void* src, const int64_t* slot, void* records, int64_t n_rows,
                     int64_t record_rows, hipStream_t s);
 int launch_kv_copy(const void* src, const int64_t* slot, void* pool, int64_t n_rows, int64_t pool_rows, hipStream_t s);
+// What the index producer writes for a selected position: the position itself, or (block_table
+// given) the physical row of the paged cache it lives in, -1 when masked.
+struct TopkPaging {
+  const int32_t* block_table;   // [n_rows / rows_per_seq, bt_stride] or null
+  int32_t bt_stride, page_size, rows_per_seq;
+  int64_t kv_rows;
+};
 int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_t* out, int n_rows,
-                        int n_cols, long long row_stride, int k, void* workspace, size_t workspace_bytes, int n_cu,
-                        hipStream_t s);
+                        int n_cols, long long row_stride, int k, const TopkPaging& paging, void* workspace,
+                        size_t workspace_bytes, int n_cu, hipStream_t s);
 size_t topk_workspace_bytes(int n_rows, int n_cols, int k, int n_cu);
 int launch_zero(void* ptr, size_t bytes, hipStream_t s);
 int launch_workspace_init(void* workspace, hipStream_t s);

@@ -170,10 +170,13 @@ __device__ __forceinline__ uint32_t key_of(float x) {
 // `want` largest wanted.  Entry i stands for index index0 + i (kWhole, kPart) or cand_idx[i]
 // (kMerge).  The answer goes to o[0 .. want) (kWhole, kMerge) or, key and index, to cand_key_out /
 // cand_idx_out[0 .. want) (kPart).
+// `bt_row` (kWhole, kMerge): null, or the page-table row of the row's sequence; the answer is then
+// written as physical rows of the paged cache (-1 where the table masks a position).
 template <int WAVES, int R, int MODE>
 __device__ __forceinline__ void resident_select(const float* __restrict__ x, int n, int want, int index0,
                                                 const int32_t* __restrict__ cand_idx, int32_t* __restrict__ o,
-                                                uint32_t* __restrict__ cand_key_out, int32_t* __restrict__ cand_idx_out) {
+                                                uint32_t* __restrict__ cand_key_out, int32_t* __restrict__ cand_idx_out,
+                                                const int32_t* __restrict__ bt_row, const TopkPaging& pg) {
   constexpr int kThreads = 64 * WAVES;
   // copies of every histogram bin, picked by lane % kCopies: score exponents are heavily skewed,
   // and lanes adding to one LDS word serialise.  A workgroup of 16 wavefronts has the LDS for one
@@ -428,9 +431,13 @@ __device__ __forceinline__ void resident_select(const float* __restrict__ x, int
   int32_t* s_list = reinterpret_cast<int32_t*>(s_raw);
   const bool staged = want <= kRawWords;
   auto emit = [&](int at, int pos) {
-    if constexpr (MODE == kWhole) o[at] = index0 + pos;
-    else if constexpr (MODE == kMerge) o[at] = cand_idx[pos];
-    else { cand_idx_out[at] = index0 + pos; cand_key_out[at] = score_key(x[pos]); }
+    if constexpr (MODE == kPart) {
+      cand_idx_out[at] = index0 + pos;
+      cand_key_out[at] = score_key(x[pos]);
+    } else {
+      const int32_t idx = MODE == kWhole ? index0 + pos : cand_idx[pos];
+      o[at] = bt_row == nullptr ? idx : paged_row(idx, bt_row, pg.bt_stride, pg.page_size, pg.kv_rows);
+    }
   };
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -472,13 +479,14 @@ template <int WAVES, int R>
 __global__ __launch_bounds__(64 * WAVES) void topk_resident_kernel(const float* __restrict__ scores,
                                                                   const int32_t* __restrict__ context_lens,
                                                                   int32_t* __restrict__ out, int n_cols,
-                                                                  long long row_stride, int k) {
+                                                                  long long row_stride, int k, TopkPaging pg) {
   const int row = blockIdx.x;
   const int n = context_lens ? max(0, min(context_lens[row], n_cols)) : n_cols;
   const int want = min(k, n);                   // entries to select
   int32_t* o = out + (size_t)row * k;
   for (int j = want + (int)threadIdx.x; j < k; j += 64 * WAVES) o[j] = -1;
-  resident_select<WAVES, R, kWhole>(scores + (size_t)row * row_stride, n, want, 0, nullptr, o, nullptr, nullptr);
+  const int32_t* bt_row = pg.block_table ? pg.block_table + (size_t)(row / pg.rows_per_seq) * pg.bt_stride : nullptr;
+  resident_select<WAVES, R, kWhole>(scores + (size_t)row * row_stride, n, want, 0, nullptr, o, nullptr, nullptr, bt_row, pg);
 }
 
 // ---- a row cut into parts ----------------------------------------------------------------------
@@ -502,14 +510,15 @@ __global__ __launch_bounds__(64 * WAVES) void topk_part_kernel(const float* __re
   const size_t base = (size_t)row * n_parts * k + before;
   const int first = part * part_len;
   resident_select<WAVES, R, kPart>(scores + (size_t)row * row_stride + first, max(0, min(n - first, part_len)), want, first, nullptr,
-                                   nullptr, cand_key + base, cand_idx + base);
+                                   nullptr, cand_key + base, cand_idx + base, nullptr, TopkPaging{});
 }
 
 template <int WAVES, int R>
 __global__ __launch_bounds__(64 * WAVES) void topk_merge_kernel(const uint32_t* __restrict__ cand_key,
                                                                const int32_t* __restrict__ cand_idx,
                                                                const int32_t* __restrict__ context_lens,
-                                                               int32_t* __restrict__ out, int n_cols, int k, int n_parts, int part_len) {
+                                                               int32_t* __restrict__ out, int n_cols, int k, int n_parts, int part_len,
+                                                               TopkPaging pg) {
   const int row = blockIdx.x;
   const int n = context_lens ? max(0, min(context_lens[row], n_cols)) : n_cols;
   int n_cand = 0;
@@ -518,7 +527,9 @@ __global__ __launch_bounds__(64 * WAVES) void topk_merge_kernel(const uint32_t* 
   int32_t* o = out + (size_t)row * k;
   for (int j = want + (int)threadIdx.x; j < k; j += 64 * WAVES) o[j] = -1;
   const size_t base = (size_t)row * n_parts * k;
-  resident_select<WAVES, R, kMerge>(reinterpret_cast<const float*>(cand_key + base), n_cand, want, 0, cand_idx + base, o, nullptr, nullptr);
+  const int32_t* bt_row = pg.block_table ? pg.block_table + (size_t)(row / pg.rows_per_seq) * pg.bt_stride : nullptr;
+  resident_select<WAVES, R, kMerge>(reinterpret_cast<const float*>(cand_key + base), n_cand, want, 0, cand_idx + base, o, nullptr, nullptr,
+                                    bt_row, pg);
 }
 
 // Rows of any length: every pass walks the row in memory.
@@ -526,7 +537,7 @@ template <int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void topk_stream_kernel(const float* __restrict__ scores,
                                                                  const int32_t* __restrict__ context_lens,
                                                                  int32_t* __restrict__ out, int n_cols,
-                                                                 long long row_stride, int k) {
+                                                                 long long row_stride, int k, TopkPaging pg) {
   constexpr int kThreads = 64 * WAVES;
   constexpr int kBatch = WAVES >= 16 ? 8 : 4;
   // 16 copies of every bin, picked by lane % 16: score exponents are heavily skewed, and 64 lanes
@@ -546,6 +557,7 @@ __global__ __launch_bounds__(64 * WAVES) void topk_stream_kernel(const float* __
   for (int j = want + tid; j < k; j += kThreads) o[j] = -1;
   if (want == 0) return;
   const bool vec = ((uintptr_t)x & 15) == 0;
+  const int32_t* bt_row = pg.block_table ? pg.block_table + (size_t)(row / pg.rows_per_seq) * pg.bt_stride : nullptr;
 
   // this wavefront's segment [seg0, seg1): whole 256-entry steps
   const int seg_len = ((n + WAVES - 1) / WAVES + 255) & ~255;
@@ -645,7 +657,8 @@ __global__ __launch_bounds__(64 * WAVES) void topk_stream_kernel(const float* __
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int eq_taken_before = min(my_rank, need_eq) - min(eq_rank, need_eq);
-      if (gt[e] || (eq[e] && my_rank < need_eq)) o[pos + gt_before + eq_taken_before] = i0 + e;
+      if (gt[e] || (eq[e] && my_rank < need_eq))
+        o[pos + gt_before + eq_taken_before] = bt_row == nullptr ? i0 + e : paged_row(i0 + e, bt_row, pg.bt_stride, pg.page_size, pg.kv_rows);
       gt_before += gt[e] ? 1 : 0;
       my_rank += eq[e] ? 1 : 0;
     }
@@ -680,8 +693,8 @@ size_t topk_workspace_bytes(int n_rows, int n_cols, int k, int n_cu) {
 }
 
 int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_t* out, int n_rows,
-                        int n_cols, long long row_stride, int k, void* workspace, size_t workspace_bytes, int n_cu,
-                        hipStream_t s) {
+                        int n_cols, long long row_stride, int k, const TopkPaging& pg, void* workspace, size_t workspace_bytes,
+                        int n_cu, hipStream_t s) {
   if (n_rows == 0) return SMLA_OK;
   int part_len = n_cols;
   const int parts = topk_parts(n_rows, n_cols, k, n_cu, &part_len);
@@ -700,11 +713,11 @@ int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_
     const dim3 grid2((unsigned)n_rows);
     const long long n_cand = (long long)parts * k;
     if (n_cand <= 4096)
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<4, 1>), grid2, dim3(256), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len);
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<4, 1>), grid2, dim3(256), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len, pg);
     else if (n_cand <= 16384)
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<16, 1>), grid2, dim3(1024), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len);
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<16, 1>), grid2, dim3(1024), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len, pg);
     else
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<16, 4>), grid2, dim3(1024), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len);
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_merge_kernel<16, 4>), grid2, dim3(1024), 0, s, cand_key, cand_idx, context_lens, out, n_cols, k, parts, part_len, pg);
     return hip_status(hipGetLastError());
   }
   const dim3 grid((unsigned)n_rows);
@@ -714,15 +727,15 @@ int launch_topk_indices(const float* scores, const int32_t* context_lens, int32_
   // latency counts: 16 wavefronts.
   const bool many = n_rows >= 1024;
   if (n_cols <= 4096)
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<4, 1>), grid, dim3(256), 0, s, scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<4, 1>), grid, dim3(256), 0, s, scores, context_lens, out, n_cols, row_stride, k, pg);
   else if (n_cols <= 16384 && many)
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<4, 4>), grid, dim3(256), 0, s, scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<4, 4>), grid, dim3(256), 0, s, scores, context_lens, out, n_cols, row_stride, k, pg);
   else if (n_cols <= 16384)
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<16, 1>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<16, 1>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k, pg);
   else if (n_cols <= 65536)
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<16, 4>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_resident_kernel<16, 4>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k, pg);
   else
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_stream_kernel<16>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(topk_stream_kernel<16>), grid, dim3(1024), 0, s, scores, context_lens, out, n_cols, row_stride, k, pg);
   return hip_status(hipGetLastError());
 }
 

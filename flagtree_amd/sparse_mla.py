@@ -353,7 +353,8 @@ def reshape_and_cache(latent, kv_cache, slot_mapping, kv_format="bf16"):
     _lib.check(rc, "smla_kv_write")
 
 
-def topk_indices(scores, k, context_lens=None, workspace=None):
+def topk_indices(scores, k, context_lens=None, workspace=None, *, block_table=None, page_size=64, kv_rows=None,
+                 rows_per_seq=1):
     """Top-k index producer: int32 [..., k] indices of the k largest entries of each row of ``scores``
     (f32 [..., N]) among its first ``context_lens[row]`` entries (default N), ascending, -1 padded.
     Ties at the k-th value go to the lower index.  The reference only has ``topk`` as a language
@@ -361,7 +362,13 @@ def topk_indices(scores, k, context_lens=None, workspace=None):
     Few long rows are cut into parts, one workgroup each, through a scratch buffer: ``workspace``
     (a uint8 device tensor of ``topk_workspace_bytes`` bytes, e.g. kept by a serving loop), or one
     allocated here for the call; ``workspace=False`` keeps one workgroup per row.  Same result
-    every way."""
+    every way.
+
+    With ``block_table`` [n_seqs, max_pages] (int32, row r belongs to sequence r // rows_per_seq) the
+    selected positions are written as physical rows of the paged cache of ``kv_rows`` rows
+    (``page_size`` positions a page; -1 where the table masks a position): a list to hand to
+    ``sparse_mla_fwd(..., block_table=None, per_sequence=False)``, which then skips its own
+    page-table look-up."""
     if not _lib.on_device(scores):
         raise ValueError("topk_indices needs device tensors (there is no CPU path)")
     if scores.dtype != torch.float32:
@@ -388,11 +395,22 @@ def topk_indices(scores, k, context_lens=None, workspace=None):
     elif workspace is not None:
         if workspace.dtype != torch.uint8 or not workspace.is_contiguous() or not _lib.on_device(workspace):
             raise ValueError("workspace must be a contiguous uint8 device tensor")
-    rc = lib.smla_topk_indices(s2.data_ptr(), cl.data_ptr() if cl is not None else None, out.data_ptr(),
-                               rows, n, s2.stride(0) if rows > 1 else n, k,
-                               workspace.data_ptr() if workspace is not None else None,
-                               workspace.numel() if workspace is not None else 0, _stream(s2))
-    _lib.check(rc, "smla_topk_indices")
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_len = workspace.numel() if workspace is not None else 0
+    if block_table is None:
+        rc = lib.smla_topk_indices(s2.data_ptr(), cl.data_ptr() if cl is not None else None, out.data_ptr(),
+                                   rows, n, s2.stride(0) if rows > 1 else n, k, ws_ptr, ws_len, _stream(s2))
+        _lib.check(rc, "smla_topk_indices")
+        return out.reshape(*lead, k)
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or not _lib.on_device(block_table):
+        raise ValueError("block_table must be an int32 device tensor [n_seqs, max_pages]")
+    if kv_rows is None or rows_per_seq <= 0 or rows % rows_per_seq != 0 or block_table.shape[0] != rows // rows_per_seq:
+        raise ValueError("with block_table: kv_rows, and one table row per rows_per_seq score rows")
+    bt = block_table.contiguous()
+    rc = lib.smla_topk_rows(s2.data_ptr(), cl.data_ptr() if cl is not None else None, bt.data_ptr(), out.data_ptr(),
+                            rows, n, s2.stride(0) if rows > 1 else n, k, rows_per_seq, page_size, bt.shape[1], int(kv_rows),
+                            ws_ptr, ws_len, _stream(s2))
+    _lib.check(rc, "smla_topk_rows")
     return out.reshape(*lead, k)
 
 

@@ -250,8 +250,25 @@ int smla_topk_indices(const float* scores, const int32_t* context_lens, int32_t*
                       int32_t n_rows, int32_t n_cols, int64_t row_stride, int32_t k, void* workspace,
                       size_t workspace_bytes, void* stream);
 
-/* Bytes of workspace with which smla_topk_indices cuts rows of this shape into parts on the current
- * device; 0 when it would not (many rows, short rows).  No counterpart in the reference. */
+/*
+ * The same selection, written as physical rows of a paged cache: entry j of rows_out[r, :] is
+ *   block_table[r / rows_per_seq, i / page_size] * page_size + i % page_size
+ * for the j-th selected position i (in ascending order of i), or -1 where the table has no page for
+ * it, the page number is negative or the row lies past kv_rows -- exactly what smla_fwd would make
+ * of position i (smla_gather_rows exposes that translation).  A list produced here goes to
+ * smla_fwd with block_table = NULL and kv_seq_stride = 0: the attention kernel then starts
+ * fetching rows one dependent memory round trip earlier (no page-table look-up of its own).
+ * block_table device int32 [n_rows / rows_per_seq, block_table_stride]; everything else as
+ * smla_topk_indices.  The reference does the look-up inside its attention kernels
+ * (/root/reference/third_party/mthreads/python/test/wmma/test_accuracy_musa_vllm_mla.py:278-283).
+ */
+int smla_topk_rows(const float* scores, const int32_t* context_lens, const int32_t* block_table,
+                   int32_t* rows_out, int32_t n_rows, int32_t n_cols, int64_t row_stride, int32_t k,
+                   int32_t rows_per_seq, int32_t page_size, int32_t block_table_stride, int64_t kv_rows,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of workspace with which smla_topk_indices / smla_topk_rows cut rows of this shape into parts on
+ * the current device; 0 when they would not (many rows, short rows).  No counterpart in the reference. */
 size_t smla_topk_workspace_bytes(int32_t n_rows, int32_t n_cols, int32_t k);
 
 /*

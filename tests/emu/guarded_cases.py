@@ -114,6 +114,11 @@ def _topk(G):
             out2 = G(torch.zeros((rows, k), dtype=torch.int32))
             assert harness.lib().smla_topk_indices(scores.data_ptr(), lens.data_ptr(), out2.data_ptr(), rows, n, n, k, ws.data_ptr(), need, None) == 0
             assert torch.equal(out, out2)
+        pages = -(-n // 64)
+        bt = G(torch.randperm(rows * pages, generator=g).to(torch.int32).view(rows, pages))
+        out3 = G(torch.zeros((rows, k), dtype=torch.int32))             # the same as physical rows through a guarded page table
+        assert harness.lib().smla_topk_rows(scores.data_ptr(), lens.data_ptr(), bt.data_ptr(), out3.data_ptr(), rows, n, n, k, 1, 64, pages,
+                                            rows * pages * 64 - 7, None, 0, None) == 0
 
 
 def _gemm(G):

@@ -838,6 +838,58 @@ def test_topk_tie_run_across_a_part_boundary():
     assert np.array_equal(to_np(out), want)
 
 
+@pytest.mark.parametrize("rows,n,k,page_size,rows_per_seq", [(4, 3000, 200, 64, 2), (2, 20000, 300, 16, 1), (3, 70001, 128, 128, 1),
+                                                             (6, 1000, 1000, 1, 3)])
+def test_topk_written_as_physical_rows(rows, n, k, page_size, rows_per_seq):
+    """smla_topk_rows = the selection followed by the page translation the attention kernels do
+    (oracle.translate_indices), bit for bit: a table that covers only part of the positions, a hole
+    (negative page number) and pages past the pool included; one workgroup per row and rows cut
+    into parts; and the attention kernel fed with the rows gives the bits it gives when it does
+    the look-up itself."""
+    lib = harness.lib()
+    g = torch.Generator().manual_seed(rows + n)
+    scores = torch.randn((rows, n), generator=g)
+    lens = torch.randint(1, n + 1, (rows,), generator=g, dtype=torch.int32)
+    n_seqs = rows // rows_per_seq
+    pages = max(1, (n * 3 // 4) // page_size)                   # the table ends before the longest contexts do
+    bt = torch.randperm(n_seqs * pages + 5, generator=g)[:n_seqs * pages].to(torch.int32).view(n_seqs, pages)
+    if pages > 2:
+        bt[0, 1] = -1
+    kv_rows = (n_seqs * pages + 2) * page_size                  # the three highest page numbers lie past the pool
+    want = oracle.translate_indices(oracle.topk_indices(to_np(scores), k, to_np(lens)), to_np(bt), page_size, kv_rows=kv_rows,
+                                    tokens_per_seq=rows_per_seq)
+    assert (want < 0).any() and (want >= 0).any()
+    need = lib.smla_topk_workspace_bytes(rows, n, k)
+    for ws_bytes in ({0, need}):
+        ws = torch.zeros(max(ws_bytes, 1), dtype=torch.uint8)
+        out = torch.full((rows, k), -9, dtype=torch.int32)
+        rc = lib.smla_topk_rows(scores.data_ptr(), lens.data_ptr(), bt.data_ptr(), out.data_ptr(), rows, n, n, k, rows_per_seq, page_size,
+                                pages, kv_rows, ws.data_ptr() if ws_bytes else None, ws_bytes, None)
+        assert rc == 0 and np.array_equal(to_np(out), want), ws_bytes
+
+
+def test_attention_over_physical_rows_from_the_index_producer():
+    from flagtree_amd import workloads
+    lib = harness.lib()
+    cfg = workloads.decode_bf16("cpu", batch=3, heads=128, pages_per_seq=6, topk=200, pad_frac=0.0)
+    B, page_size, pages = 3, cfg["page_size"], cfg["block_table"].shape[1]
+    n, k = pages * page_size, 200
+    g = torch.Generator().manual_seed(3)
+    scores = torch.randn((B, n), generator=g)
+    lens = torch.tensor([n, n // 2, 150], dtype=torch.int32)
+    kv_rows = cfg["kv_cache"].numel() // 576
+    logical = torch.full((B, k), -9, dtype=torch.int32)
+    rows = torch.full((B, k), -9, dtype=torch.int32)
+    assert lib.smla_topk_indices(scores.data_ptr(), lens.data_ptr(), logical.data_ptr(), B, n, n, k, None, 0, None) == 0
+    assert lib.smla_topk_rows(scores.data_ptr(), lens.data_ptr(), cfg["block_table"].data_ptr(), rows.data_ptr(), B, n, n, k, 1, page_size,
+                              pages, kv_rows, None, 0, None) == 0
+    out0, lse0, rc0 = harness.forward(dict(cfg, indices=logical.view(B, 1, k)), n_splits=2)
+    out1, lse1, rc1 = harness.forward(dict(cfg, indices=rows.view(B, 1, k), block_table=None, kv_cache=cfg["kv_cache"].reshape(-1, 576)), n_splits=2)
+    assert rc0 == 0 and rc1 == 0
+    assert torch.equal(out0.view(torch.int16), out1.view(torch.int16)) and torch.equal(lse0, lse1)
+    _check(dict(cfg, indices=logical.view(B, 1, k)), out1, lse1)
+
+
 def test_topk_part_planning():
     lib = harness.lib()
     try:

@@ -330,6 +330,51 @@ def test_topk_indices_degenerate_rows(dev, n, k):
         assert np.array_equal(to_np(got1), oracle.topk_indices(x, k))
 
 
+@pytest.mark.parametrize("rows,n,k,page_size,rows_per_seq", [(4, 3000, 200, 64, 2), (8, 65536, 2048, 64, 1), (6, 1000, 1000, 1, 3)])
+def test_topk_written_as_physical_rows(dev, rows, n, k, page_size, rows_per_seq):
+    """The index producer's list as physical rows of the paged cache = its list of positions put
+    through the translation of the attention kernels (oracle.translate_indices), bit for bit, with a
+    table shorter than the contexts, a hole and pages past the pool."""
+    import flagtree_amd as ft
+    g = torch.Generator().manual_seed(rows + n)
+    scores = torch.randn((rows, n), generator=g)
+    lens = torch.randint(1, n + 1, (rows,), generator=g, dtype=torch.int32)
+    n_seqs = rows // rows_per_seq
+    pages = max(1, (n * 3 // 4) // page_size)
+    bt = torch.randperm(n_seqs * pages + 5, generator=g)[:n_seqs * pages].to(torch.int32).view(n_seqs, pages)
+    if pages > 2:
+        bt[0, 1] = -1
+    kv_rows = (n_seqs * pages + 2) * page_size
+    want = oracle.translate_indices(oracle.topk_indices(scores.numpy(), k, lens.numpy()), bt.numpy(), page_size, kv_rows=kv_rows,
+                                    tokens_per_seq=rows_per_seq)
+    for ws in (None, False):
+        got = ft.topk_indices(scores.to(dev), k, lens.to(dev), workspace=ws, block_table=bt.to(dev), page_size=page_size,
+                              kv_rows=kv_rows, rows_per_seq=rows_per_seq)
+        assert np.array_equal(to_np(got), want)
+
+
+def test_attention_over_physical_rows_from_the_index_producer(dev):
+    """Rows from the index producer, no page table for the attention kernel: the same bits as
+    positions plus page table."""
+    import flagtree_amd as ft
+    from flagtree_amd import workloads
+    cfg = workloads.decode_bf16(dev, batch=6, heads=128, pages_per_seq=24, topk=512, pad_frac=0.0)
+    B, page_size, pages = 6, cfg["page_size"], cfg["block_table"].shape[1]
+    n, k = pages * page_size, 512
+    g = torch.Generator().manual_seed(3)
+    scores = torch.randn((B, n), generator=g).to(dev)
+    lens = torch.tensor([n, n // 2, 150, n, 700, n - 1], dtype=torch.int32).to(dev)
+    kv_rows = cfg["kv_cache"].numel() // 576
+    logical = ft.topk_indices(scores, k, lens)
+    rows = ft.topk_indices(scores, k, lens, block_table=cfg["block_table"], page_size=page_size, kv_rows=kv_rows)
+    out0, lse0 = _fwd(dict(cfg, indices=logical.view(B, 1, k)), n_splits=2)
+    out1, lse1 = ft.sparse_mla_fwd(cfg["q"], cfg["kv_cache"].reshape(-1, 576), rows.view(B, 1, k), cfg["sm_scale"], 512,
+                                   kv_format="bf16", n_splits=2, per_sequence=False)
+    torch.cuda.synchronize()
+    assert torch.equal(out0, out1) and torch.equal(lse0, lse1)
+    _check(dict(cfg, indices=logical.view(B, 1, k)), out1, lse1)
+
+
 def test_topk_feeds_sparse_mla(dev):
     """Indexer scores -> top-k indices -> sparse attention: same result as handing the oracle's
     index list to the attention kernel."""

@@ -86,6 +86,11 @@ def test_validation_codes_without_a_device(lib):
     assert lib.smla_topk_indices(p16, None, p16, 1, 0, 64, 8, None, 0, None) == -2 and lib.smla_topk_indices(p16, None, p16, 1, 64, 64, 0, None, 0, None) == -2
     assert lib.smla_topk_indices(p16, None, p16, -1, 64, 64, 8, None, 0, None) == -2
     assert lib.smla_topk_indices(p16, None, p16, 1, 64, 32, 8, None, 0, None) == -2                   # row stride shorter than a row
+    assert lib.smla_topk_indices(p16, None, p16, 1, 64, 64, 8, p16 + 2, 64, None) == -3               # workspace off a 4-byte boundary
+    assert lib.smla_topk_rows(p16, None, None, p16, 2, 64, 64, 8, 1, 16, 4, 100, None, 0, None) == -1   # no page table
+    assert lib.smla_topk_rows(p16, None, p16, p16, 3, 64, 64, 8, 2, 16, 4, 100, None, 0, None) == -2    # rows do not divide into sequences
+    assert lib.smla_topk_rows(p16, None, p16, p16, 2, 64, 64, 8, 1, 0, 4, 100, None, 0, None) == -2     # page size
+    assert lib.smla_topk_rows(p16, None, p16, p16, 2, 64, 64, 8, 1, 16, 4, 0, None, 0, None) == -2      # empty pool
 
     def dense(**kw):
         a = dict(ok, **kw)
