@@ -16,6 +16,8 @@
 // X rows it re-reads stay in its L2.
 #include "smla_common.h"
 
+#include <stdlib.h>
+
 namespace smla {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 g_bf16x8;
@@ -235,14 +237,27 @@ __device__ __forceinline__ g_bf16x4 g_lds_tr(uint32_t a) {
   return hw::lds_read_tr16_b64(a);
 }
 
+// What a persistent workgroup carries from one tile to the next (CHAIN): which of the two K-step
+// buffers holds, or is receiving, K-step 0 of the current tile, whether the tile before has already
+// sent for it, and where the next tile lies, so that this tile can send for the next one's K-step 0
+// during its own last K-step.  The next tile's first fetch then runs under this tile's epilogue,
+// which for that reason stages through ONE buffer (the one the last K-step was read from), 16 rows
+// of a wavefront's block at a time, while the other buffer receives.
+struct TileChain {
+  int base;
+  bool primed, has_next;
+  int next_m0, next_n0;
+};
+
 // One output tile of 128 MI rows x 256 columns (MI = 2: the full 256 x 256 tile; MI = 1: its upper
 // or lower half, used to fill the last, partly occupied round of tiles, see launch_gemm_rs).
 // Wavefront (wm, wn) owns rows 32 MI wm .. + 32 MI - 1 and columns 64 wn .. + 63.
-template <int MI>
+template <int MI, bool CHAIN = false>
 __device__ __forceinline__ void gemm_big_tile(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                               const float* __restrict__ partial, uint16_t* __restrict__ out, int N, int K,
                                               int rows_per_chunk, long long chunk_stride, int m0, int n0,
-                                              uint8_t* s_buf0) {
+                                              uint8_t* s_buf0, TileChain* chain = nullptr) {
+  static_assert(!CHAIN || MI == 2, "only whole tiles are chained");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 2, wn = wave & 3;
@@ -264,26 +279,28 @@ __device__ __forceinline__ void gemm_big_tile(const uint16_t* __restrict__ x, co
 #pragma unroll
     for (int odd = 0; odd < 2; ++odd) {
       const int blk = (pb >> 2) ^ ((2 * odd + kl) & 3); // row k = 2 i + kl: k & 3 = (2 i + kl) & 3
-      b_off[odd] = (uint32_t)((kl * N + n0 + 8 * (4 * blk + (pb & 3))) * 2);
+      b_off[odd] = (uint32_t)((kl * N + 8 * (4 * blk + (pb & 3))) * 2);
     }
   }
-  // DMA slot d = 0..3 of this wavefront for the K-step at k0 into buffer buf (0, 1: X, 2, 3: W)
-  auto issue_dma = [&](int d, int k0, int buf) {
+  // DMA slot d = 0..3 of this wavefront for the K-step at k0 of the tile at (tm0, tn0) into buffer buf (0, 1: X, 2, 3: W)
+  auto issue_dma_at = [&](int d, int k0, int buf, int tm0, int tn0) {
     const uint32_t dst = lds0 + buf * kStage2;
     if (d < 2) {
       if (d < MI) {
         const int i = MI * wave + d;
-        const uint64_t sa = (uint64_t)(uintptr_t)x + ((uint64_t)(m0 + 8 * i) * K + k0) * 2;
+        const uint64_t sa = (uint64_t)(uintptr_t)x + ((uint64_t)(tm0 + 8 * i) * K + k0) * 2;
         const uint32_t ma = dst + i * 1024;
         hw::dma_b128(a_off[i & 1], sa, ma);
       }
     } else {
       const int i = 2 * wave + d - 2;
-      const uint64_t sb = (uint64_t)(uintptr_t)w + (uint64_t)(k0 + 2 * i) * N * 2;
+      const uint64_t sb = (uint64_t)(uintptr_t)w + ((uint64_t)(k0 + 2 * i) * N + tn0) * 2;
       const uint32_t mb = dst + kA2Bytes + i * 1024;
       hw::dma_b128(b_off[d & 1], sb, mb);
     }
   };
+  auto issue_dma = [&](int d, int k0, int buf) { issue_dma_at(d, k0, buf, m0, n0); };
+  const int base = CHAIN ? chain->base : 0;               // the buffer of this tile's K-step 0
 
   g_f32x16 acc[MI][2];
 #pragma unroll
@@ -300,8 +317,10 @@ __device__ __forceinline__ void gemm_big_tile(const uint16_t* __restrict__ x, co
   const uint32_t b_sw = (uint32_t)((l16 >> 2) & 3);
 
   const int n_k = K / kBK;
+  if (!CHAIN || !chain->primed) {
 #pragma unroll
-  for (int d = 0; d < 4; ++d) issue_dma(d, 0, 0);
+    for (int d = 0; d < 4; ++d) issue_dma(d, 0, base);
+  }
   auto load_frags = [&](uint32_t buf, int ks, g_bf16x8 (&af)[MI], g_bf16x8 (&bf)[2]) {
 #pragma unroll
     for (int i = 0; i < MI; ++i) af[i] = g_lds_b128(buf + a_lane + i * (32 * 128) + (((2 * ks + g) ^ a_sw) << 4));
@@ -316,15 +335,16 @@ __device__ __forceinline__ void gemm_big_tile(const uint16_t* __restrict__ x, co
   for (int kt = 0; kt < n_k; ++kt) {
     hw::wait_vmcnt<0>();    // this wavefront's share of step kt has landed
     __syncthreads();                                    // ... everyone's has, and everyone is done with step kt - 1
-    const uint32_t buf = lds0 + (kt & 1) * kStage2;
+    const uint32_t buf = lds0 + ((base + kt) & 1) * kStage2;
     const bool more = kt + 1 < n_k;
-    const int k_next = (kt + 1) * kBK, buf_next = (kt + 1) & 1;
+    const int k_next = (kt + 1) * kBK, buf_next = (base + kt + 1) & 1;
     g_bf16x8 af[2][MI], bf[2][2];
     load_frags(buf, 0, af[0], bf[0]);
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
       if (ks + 1 < kBK / 16) load_frags(buf, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
       if (more) issue_dma(ks, k_next, buf_next);
+      else if (CHAIN && chain->has_next) issue_dma_at(ks, 0, buf_next, chain->next_m0, chain->next_n0);   // the next tile's K-step 0
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -333,83 +353,139 @@ __device__ __forceinline__ void gemm_big_tile(const uint16_t* __restrict__ x, co
     }
   }
   __syncthreads();                                      // the buffers are free: the epilogue stages through them
+                                                        // (CHAIN: the buffer of the last K-step is; the other one is receiving)
 
-  // ---- epilogue: a wavefront parks 32 rows x 64 columns (one row of its MFMA tiles) in LDS and
+  // ---- epilogue: a wavefront parks kRowsStage rows x 64 columns of its MFMA tiles in LDS and
   // reads them back four rows a pass, four consecutive columns per lane
-  float* stage = reinterpret_cast<float*>(s_buf0) + wave * 32 * kStage2Floats;
+  constexpr int kRowsStage = CHAIN ? 16 : 32;           // rows parked at a time: 32 = a whole row of MFMA tiles
+  const int last_buf = (base + n_k - 1) & 1;
+  float* stage = CHAIN ? reinterpret_cast<float*>(s_buf0 + last_buf * kStage2) + wave * kRowsStage * kStage2Floats
+                       : reinterpret_cast<float*>(s_buf0) + wave * kRowsStage * kStage2Floats;
+  static_assert(16 * 16 * kStage2Floats * 4 <= kStage2, "chained tiles stage through one buffer");
   const int col4 = 4 * l16, rsub = lane >> 4;           // this lane's 4 columns within the wave's 64, row within a pass
   const int n = n0 + 64 * wn + col4;
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
-    g_f32x4 z[8];                                       // partial sums of rows 32*i + 4*p + rsub, p < 8
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      const int m = m0 + 32 * MI * wm + 32 * i + 4 * p + rsub;
-      z[p] = partial ? __builtin_nontemporal_load(reinterpret_cast<const g_f32x4*>(partial + (size_t)m * N + n))
-                     : g_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < 32 / kRowsStage; ++h) {         // the rows 32 i + kRowsStage h .. of the wavefront's block
+      constexpr int kPasses = kRowsStage / 4;
+      g_f32x4 z[kPasses];                               // partial sums of rows 32 i + kRowsStage h + 4 p + rsub
+#pragma unroll
+      for (int p = 0; p < kPasses; ++p) {
+        const int m = m0 + 32 * MI * wm + 32 * i + kRowsStage * h + 4 * p + rsub;
+        z[p] = partial ? __builtin_nontemporal_load(reinterpret_cast<const g_f32x4*>(partial + (size_t)m * N + n))
+                       : g_f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r >> 2) + 4 * g + (r & 3);
+        if ((8 * (r >> 2)) / kRowsStage != h) continue; // (known at compile time: 4 g + r % 4 never crosses a multiple of 8)
+#pragma unroll
+        // (a row is exactly the 64 banks wide, and a store's two half-wavefronts write rows 4 apart:
+        // rows with bit 2 set keep their two 32-float halves swapped, so the halves land on different banks)
+        for (int j = 0; j < 2; ++j) stage[(row - kRowsStage * h) * kStage2Floats + ((32 * j + c32) ^ (32 * g))] = acc[i][j][r];
+      }
+      __builtin_amdgcn_wave_barrier();                  // (the area is the wavefront's own; its LDS operations complete in order)
+#pragma unroll
+      for (int p = 0; p < kPasses; ++p) {
+        const int row = 4 * p + rsub;
+        const int m = m0 + 32 * MI * wm + 32 * i + kRowsStage * h + row;
+        const float4 v = *reinterpret_cast<const float4*>(stage + row * kStage2Floats + (col4 ^ (32 * ((row >> 2) & 1))));
+        const g_f32x4 zz = z[p];
+        const int chunk = m / rows_per_chunk;
+        uint16_t* o = out + (size_t)chunk * chunk_stride + (size_t)(m - chunk * rows_per_chunk) * N + n;
+        uint2 pk;
+        pk.x = g_pack_bf16(v.x + zz[0], v.y + zz[1]);
+        pk.y = g_pack_bf16(v.z + zz[2], v.w + zz[3]);
+        *reinterpret_cast<uint2*>(o) = pk;
+      }
+      __builtin_amdgcn_wave_barrier();
     }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 8 * (r >> 2) + 4 * g + (r & 3);
-#pragma unroll
-      // (a row is exactly the 64 banks wide, and a store's two half-wavefronts write rows 4 apart:
-      // rows with bit 2 set keep their two 32-float halves swapped, so the halves land on different banks)
-      for (int j = 0; j < 2; ++j) stage[row * kStage2Floats + ((32 * j + c32) ^ (32 * g))] = acc[i][j][r];
-    }
-    __builtin_amdgcn_wave_barrier();                    // (the area is the wavefront's own; its LDS operations complete in order)
-#pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      const int row = 4 * p + rsub;
-      const int m = m0 + 32 * MI * wm + 32 * i + row;
-      const float4 v = *reinterpret_cast<const float4*>(stage + row * kStage2Floats + (col4 ^ (32 * ((row >> 2) & 1))));
-      const g_f32x4 zz = z[p];
-      const int chunk = m / rows_per_chunk;
-      uint16_t* o = out + (size_t)chunk * chunk_stride + (size_t)(m - chunk * rows_per_chunk) * N + n;
-      uint2 pk;
-      pk.x = g_pack_bf16(v.x + zz[0], v.y + zz[1]);
-      pk.y = g_pack_bf16(v.z + zz[2], v.w + zz[3]);
-      *reinterpret_cast<uint2*>(o) = pk;
-    }
-    __builtin_amdgcn_wave_barrier();
+  }
+  if constexpr (CHAIN) {                                // hand the buffers on: the next tile's K-step 0 is on its way into the other one
+    chain->base = last_buf ^ 1;
+    chain->primed = chain->has_next;
   }
 }
 
 // Blocks [0, n_full) take whole 256 x 256 tiles; blocks from n_full on take half tiles (128 rows),
 // two consecutive blocks of an XCD the two halves of one tile.  The hardware hands out blocks in
 // id order, so the half tiles are what runs last.
+// Block id -> tile.  XCD x (= id % 8) owns m-tiles [x * mt/8, (x+1) * mt/8) when mt divides by 8.
+// Returns false for an id without a tile.
+__device__ __forceinline__ bool big_tile_of(int id, int n_full, int mt, int nt, int& tile_m, int& tile_n, int& half, bool& halves) {
+  halves = id >= n_full;
+  half = 0;
+  int xcd = id & 7, local = id >> 3;
+  if (halves) {                                         // (only with the banded mapping; n_full is a multiple of 8)
+    const int j = id - n_full;
+    xcd = j & 7;
+    half = (j >> 3) & 1;
+    local = (n_full >> 3) + (j >> 4);
+  }
+  if (mt % 8 == 0) {
+    const int band = mt / 8;
+    tile_m = xcd * band + local % band;
+    tile_n = local / band;
+  } else {
+    tile_m = id % mt;
+    tile_n = id / mt;
+  }
+  return tile_m < mt && tile_n < nt;
+}
+
 __global__ __launch_bounds__(1024)
 void gemm_rs_big_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                         const float* __restrict__ partial, uint16_t* __restrict__ out, int M, int N, int K,
                         int rows_per_chunk, long long chunk_stride, int n_full) {
   __shared__ __attribute__((aligned(1024))) uint8_t s_buf[2][kStage2];
-
-  // tile mapping: XCD x owns m-tiles [x * mt/8, (x+1) * mt/8) when mt divides by 8
   const int mt = M / kBM2, nt = N / kBN2;
-  const bool halves = (int)blockIdx.x >= n_full;
-  int tile_m, tile_n, half = 0;
-  {
-    int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    if (halves) {                                       // (only with the banded mapping; n_full is a multiple of 8)
-      const int j = (int)blockIdx.x - n_full;
-      xcd = j & 7;
-      half = (j >> 3) & 1;
-      local = (n_full >> 3) + (j >> 4);
-    }
-    if (mt % 8 == 0) {
-      const int band = mt / 8;
-      tile_m = xcd * band + local % band;
-      tile_n = local / band;
-    } else {
-      tile_m = blockIdx.x % mt;
-      tile_n = blockIdx.x / mt;
-    }
-  }
-  if (tile_m >= mt || tile_n >= nt) return;
+  int tile_m, tile_n, half;
+  bool halves;
+  if (!big_tile_of((int)blockIdx.x, n_full, mt, nt, tile_m, tile_n, half, halves)) return;
   const int n0 = tile_n * kBN2;
   if (halves)
     gemm_big_tile<1>(x, w, partial, out, N, K, rows_per_chunk, chunk_stride, tile_m * kBM2 + 128 * half, n0, &s_buf[0][0]);
   else
     gemm_big_tile<2>(x, w, partial, out, N, K, rows_per_chunk, chunk_stride, tile_m * kBM2, n0, &s_buf[0][0]);
+}
+
+// The same tiles by persistent workgroups, one per compute unit (opt-in: FLAGTREE_SMLA_GEMM_CHAIN=1).
+// Workgroup b takes the block ids b, b + gridDim.x, ... of the kernel above (gridDim.x a multiple
+// of 8, so all of them belong to its own XCD's band); its whole tiles are chained: the moves of the
+// next tile's K-step 0 go out during the current tile's last K-step and land while the epilogue
+// (partial sums in, bf16 out: traffic that otherwise finds the CU's matrix cores and its LDS
+// moves idle) runs.  Its half tiles, which come last, run one by one.
+__global__ __launch_bounds__(1024)
+void gemm_rs_chain_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                          const float* __restrict__ partial, uint16_t* __restrict__ out, int M, int N, int K,
+                          int rows_per_chunk, long long chunk_stride, int n_full, int n_ids) {
+  __shared__ __attribute__((aligned(1024))) uint8_t s_buf[2][kStage2];
+  const int mt = M / kBM2, nt = N / kBN2;
+  const int step = (int)gridDim.x;
+  TileChain chain{0, false, false, 0, 0};
+  int id = (int)blockIdx.x;
+  int tile_m, tile_n, half;
+  bool halves;
+  // whole tiles (ids below n_full; every such id has a tile when the banded mapping applies, which the launcher checks)
+  for (; id < n_full; id += step) {
+    big_tile_of(id, n_full, mt, nt, tile_m, tile_n, half, halves);
+    const int m0 = tile_m * kBM2, n0 = tile_n * kBN2;
+    chain.has_next = id + step < n_full;
+    if (chain.has_next) {
+      int nm, nn, nh;
+      bool nhalves;
+      big_tile_of(id + step, n_full, mt, nt, nm, nn, nh, nhalves);
+      chain.next_m0 = nm * kBM2;
+      chain.next_n0 = nn * kBN2;
+    }
+    gemm_big_tile<2, true>(x, w, partial, out, N, K, rows_per_chunk, chunk_stride, m0, n0, &s_buf[0][0], &chain);
+  }
+  for (; id < n_ids; id += step) {
+    __syncthreads();                                    // every wavefront is done with the tile before: its staging area is free
+    if (!big_tile_of(id, n_full, mt, nt, tile_m, tile_n, half, halves)) continue;
+    gemm_big_tile<1>(x, w, partial, out, N, K, rows_per_chunk, chunk_stride, tile_m * kBM2 + 128 * half, tile_n * kBN2, &s_buf[0][0]);
+  }
 }
 
 // How many of the 256 x 256 tiles are computed whole; the rest, the last and only partly filled
@@ -440,6 +516,15 @@ int launch_gemm_rs(const void* x, const void* w, const float* partial, void* out
     long long n_full = gemm_full_tiles(mt, nt, n_cu);
     if (n_full < tiles) blocks = n_full + 2 * (tiles - n_full);   // (only with mt a multiple of 8: blocks was mt * nt)
     else n_full = blocks;                                         // no half tiles
+    // persistent workgroups (opt-in): needs the banded mapping with every id a tile, and a workgroup count that keeps ids on their XCD
+    const char* e = getenv("FLAGTREE_SMLA_GEMM_CHAIN");
+    if (e != nullptr && e[0] == '1' && mt % 8 == 0 && n_cu % 8 == 0 && blocks > n_cu) {
+      if (n_full == blocks) n_full = tiles;                       // (mt % 8 == 0: blocks == tiles)
+      hipLaunchKernelGGL(gemm_rs_chain_kernel, dim3((unsigned)n_cu), dim3(1024), 0, s,
+          static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), partial, static_cast<uint16_t*>(out), m, n, k,
+          m / n_chunks, (long long)chunk_stride, (int)n_full, (int)blocks);
+      return hip_status(hipGetLastError());
+    }
     hipLaunchKernelGGL(gemm_rs_big_kernel, dim3((unsigned)blocks), dim3(1024), 0, s,
         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w), partial, static_cast<uint16_t*>(out), m, n, k,
         m / n_chunks, (long long)chunk_stride, (int)n_full);

@@ -144,7 +144,7 @@ def topk_case(seed, rng, g, end):
 def gemm_case(seed, rng, g, end):
     lib = harness.lib()
     m = int(rng.choice([128, 256, 384, 512, 2048]))
-    n = int(rng.choice([256, 512, 768]))
+    n = int(rng.choice([256, 512, 768, 1280]))
     k = int(rng.choice([64, 128, 192]))
     chunks = int(rng.choice([c for c in (1, 2, 4, 8) if m % c == 0]))
     extra = int(rng.choice([0, 8, 64]))
@@ -156,7 +156,11 @@ def gemm_case(seed, rng, g, end):
     part = G(pt, end).tensor if use_p else None
     out = G(torch.full((chunks * stride,), float("nan"), dtype=torch.bfloat16), end).tensor
     cus = int(rng.choice([16, 16, 20, 256]))                # 20: no multiple of 8, so no half tiles
-    print(f"seed {seed} gemm m={m} n={n} k={k} chunks={chunks} stride_extra={extra} partial={use_p} cus={cus}", flush=True)
+    os.environ.pop("FLAGTREE_SMLA_GEMM_CHAIN", None)
+    if rng.random() < 0.5:
+        os.environ["FLAGTREE_SMLA_GEMM_CHAIN"] = "1"        # persistent workgroups (where the shape has more tiles than units)
+    print(f"seed {seed} gemm m={m} n={n} k={k} chunks={chunks} stride_extra={extra} partial={use_p} cus={cus} "
+          f"chain={'FLAGTREE_SMLA_GEMM_CHAIN' in os.environ}", flush=True)
     random_schedule(rng)
     try:
         lib.emu_set_cu_count(cus)

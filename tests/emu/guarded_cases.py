@@ -130,6 +130,18 @@ def _gemm(G):
         out = G(torch.zeros((m, n), dtype=torch.bfloat16))
         assert harness.lib().smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), partial.data_ptr(), out.data_ptr(), m, n, k, chunks,
                                                 (m // chunks) * n, None) == 0
+    # persistent workgroups chaining two whole tiles each, then a half tile (40 tiles on 16 compute units)
+    os.environ["FLAGTREE_SMLA_GEMM_CHAIN"] = "1"
+    try:
+        m, n, k, chunks = 2048, 1280, 192, 4
+        x = G((torch.randn((m, k), generator=g) * 0.1).to(torch.bfloat16))
+        w = G((torch.randn((k, n), generator=g) * 0.1).to(torch.bfloat16))
+        partial = G(torch.randn((m, n), generator=g))
+        out = G(torch.zeros((m, n), dtype=torch.bfloat16))
+        assert harness.lib().smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), partial.data_ptr(), out.data_ptr(), m, n, k, chunks,
+                                                (m // chunks) * n, None) == 0
+    finally:
+        os.environ.pop("FLAGTREE_SMLA_GEMM_CHAIN")
 
 
 def _merge(G):

@@ -924,6 +924,36 @@ def test_local_gemm(m, n, k, chunks):
     harness.configure()
 
 
+@pytest.mark.parametrize("m,n,k,chunks", [(2048, 1280, 128, 2),     # 40 tiles on 16 units: two whole tiles chained per workgroup, then a half tile
+                                          (2048, 1280, 192, 8),     # three K-steps: the buffers swap roles from tile to tile
+                                          (2048, 1024, 64, 1),      # one K-step a tile, 32 tiles: two chained whole tiles, no halves
+                                          (4096, 1536, 128, 4),     # 96 tiles: six chained whole tiles per workgroup
+                                          (2048, 768, 128, 2)])     # 24 tiles: one whole tile and one half tile per workgroup
+def test_local_gemm_by_persistent_workgroups(m, n, k, chunks, monkeypatch):
+    """FLAGTREE_SMLA_GEMM_CHAIN=1: one workgroup per compute unit walks its tiles; the next tile's
+    first K-step is sent for during the current tile's last one and lands under the epilogue, which
+    stages through the other buffer.  Same bits as one workgroup per tile (every output element is
+    the same sum in the same order), under in-step, skewed and eager-move schedules."""
+    g = torch.Generator().manual_seed(m + n + k)
+    x = (torch.randn((m, k), generator=g) * 0.1).to(torch.bfloat16)
+    w = (torch.randn((k, n), generator=g) * 0.1).to(torch.bfloat16)
+    partial = torch.randn((m, n), generator=g)
+    lib = harness.lib()
+    ref = torch.full((m, n), float("nan"), dtype=torch.bfloat16)
+    assert lib.smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), partial.data_ptr(), ref.data_ptr(), m, n, k, chunks, (m // chunks) * n, None) == 0
+    monkeypatch.setenv("FLAGTREE_SMLA_GEMM_CHAIN", "1")
+    for eager, skew, together in ((False, 0, 0), (True, 0, 0), (False, 1, 0), (True, 2, 3)):
+        harness.configure(dma_eager=eager, wave_skew_seed=skew, concurrent_blocks=together, concurrent_seed=4)
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16)
+        launches, before = lib.emu_launch_count(), harness.work_counts()
+        rc = lib.smla_gemm_rs_local(x.data_ptr(), w.data_ptr(), partial.data_ptr(), out.data_ptr(), m, n, k, chunks, (m // chunks) * n, None)
+        assert rc == 0 and harness.work_counts()["mfma_flops"] == 2.0 * m * n * k
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), (eager, skew)
+    harness.configure()
+    want = oracle.gemm_rs_local(to_np(x), to_np(w), to_np(partial), n_chunks=chunks).reshape(m, n)
+    assert max_abs(to_np(out), want) <= 1e-2 + 1e-2 * float(np.abs(want).max())
+
+
 def test_local_gemm_on_a_compute_unit_count_that_is_no_multiple_of_eight():
     """24 tiles on 20 compute units leave a rest of 4 tiles, few enough to be halved; but the half-tile
     mapping needs the whole tiles to come in groups of 8, which 20 does not give: all tiles stay

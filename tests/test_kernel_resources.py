@@ -19,7 +19,9 @@ LDS_PER_CU = 160 * 1024
 #    per-chunk set-up.
 #  * the wavefront-per-head-group kernel holds 144 Q and 256 accumulator registers; it parks values
 #    across the per-chunk set-up and in the epilogue's merge.
-MAY_SPILL = ("fwd_few_fp8_kernel", "fwd_group_kernel")
+#  * the persistent GEMM kernel holds the whole-tile and the half-tile code; four lane-derived
+#    offsets of the half-tile part are parked at the kernel's start and fetched once, before it.
+MAY_SPILL = ("fwd_few_fp8_kernel", "fwd_group_kernel", "gemm_rs_chain_kernel")
 
 _cache = {}
 
