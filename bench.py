@@ -51,6 +51,9 @@ def parse():
     ap.add_argument("--fp8-mfma", action="store_true",
                     help="decode_fp8 on the kernel that contracts the records' e4m3 codes with fp8 MFMAs (sets "
                          "FLAGTREE_SMLA_FP8_MFMA=1; opt-in until measured)")
+    ap.add_argument("--persist", action="store_true",
+                    help="unsplit many-heads launches (prefill_causal_bf16, decode_dense_bf16) by one persistent workgroup per "
+                         "compute unit (sets FLAGTREE_SMLA_PERSIST=1; opt-in until measured)")
     ap.add_argument("--topk-one-workgroup", action="store_true",
                     help="topk_* workloads: one workgroup per row even where the rows would be cut into parts")
     ap.add_argument("--token-bands", action="store_true",
@@ -145,6 +148,8 @@ def main():
         os.environ["FLAGTREE_SMLA_FEW_FP8"] = "1"
     if a.fp8_mfma:
         os.environ["FLAGTREE_SMLA_FP8_MFMA"] = "1"
+    if a.persist:
+        os.environ["FLAGTREE_SMLA_PERSIST"] = "1"
     if a.head_groups:
         os.environ["FLAGTREE_SMLA_HEAD_GROUPS"] = "1"
     if a.token_bands:
@@ -279,7 +284,7 @@ def main():
         roof = dict(bound="mfma", achieved=flops / (kern_ms * 1e-3) / 1e12, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
     # (the stored counter figures were taken on the default kernels: none for a kernel behind a switch)
-    roof["traffic"] = None if (a.head_groups or a.few_fp8 or a.fp8_mfma or a.token_bands) else measured_traffic(a.workload)
+    roof["traffic"] = None if (a.head_groups or a.few_fp8 or a.fp8_mfma or a.token_bands or a.persist) else measured_traffic(a.workload)
     roof["traffic_source"] = TRAFFIC_NOTE
     roof["kernel"] = many_heads_kernel(a, fmt) if H > 32 else ("fwd_few_f8_kernel" if a.fp8_mfma and hbm_bound else "fwd_few_fp8_kernel" if a.few_fp8 and hbm_bound else "fwd_short_kernel")
     roof["kernel_ms"] = kern_ms
@@ -464,7 +469,7 @@ def bench_dense(a, torch, ft, workloads, dev):
         "config": {"workload": "decode_dense_bf16", "batch": B, "heads": H, "context": ctx, "page_size": cfg["page_size"],
                    "flops_per_step": flops, "bytes_per_step": nbytes},
         "roofline": {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": ach / PEAK_BF16_TFLOPS, "traffic": None if a.head_groups else measured_traffic("decode_dense_bf16"),
+                     "frac": ach / PEAK_BF16_TFLOPS, "traffic": None if (a.head_groups or a.persist) else measured_traffic("decode_dense_bf16"),
                      "traffic_source": TRAFFIC_NOTE, "kernel": many_heads_kernel(a, "bf16"), "kernel_ms": kern_ms,
                      "other_bound": {"bound": "hbm", "achieved": nbytes / (kern_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                                      "unit": "GB/s", "frac": nbytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}},

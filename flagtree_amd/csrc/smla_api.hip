@@ -43,6 +43,14 @@ bool few_fp8_enabled() {
 // FLAGTREE_SMLA_FP8_MFMA=1 sends few-heads launches over an fp8 cache to the kernel that contracts
 // the records' e4m3 codes on the matrix cores as they are (smla_mfma_few_f8.hip; also two
 // workgroups per CU).  It wins over FLAGTREE_SMLA_FEW_FP8.
+// FLAGTREE_SMLA_PERSIST=1: many-heads launches that do not split and have at least two items per
+// compute unit (prefill, dense decode over many tokens) run one persistent workgroup per compute
+// unit, which sends for the next item's indices and Q under the current item's epilogue.
+bool persist_enabled() {
+  const char* e = getenv("FLAGTREE_SMLA_PERSIST");
+  return e != nullptr && e[0] == '1';
+}
+
 bool fp8_mfma_enabled() {
   const char* e = getenv("FLAGTREE_SMLA_FP8_MFMA");
   return e != nullptr && e[0] == '1';
@@ -180,6 +188,7 @@ static int fill_params(Params& p, const void* q, const void* kv, const int32_t* 
   p.kv_seq_stride = kv_seq_stride; p.kv_rows = kv_rows; p.sm_scale = sm_scale; p.logit_cap = 0.f;
   p.token_band = token_bands_enabled() ? (n_tokens + 7) / 8 : 0;
   p.merge_in_launch = 0;
+  p.persist_workgroups = 0;
   return SMLA_OK;
 }
 
@@ -228,6 +237,7 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
     p.part_lse = p.part_out + (size_t)n_tokens * n_splits * n_heads * d_v;
     p.merge_in_launch = merge_in_launch_ok() ? 1 : 0;
   }
+  if (persist_enabled() && device_cus() % 8 == 0) p.persist_workgroups = device_cus();
   if (n_heads > 32 && head_groups_enabled()) rc = launch_fwd_group(kv_format, p, s);
   else if (n_heads > 32) rc = launch_fwd_tall(kv_format, p, s);
   else if (kv_format == SMLA_KV_FP8_B128 && fp8_mfma_enabled()) rc = launch_fwd_few_f8(p, s);

@@ -35,6 +35,7 @@ struct Params {
   float sm_scale;
   float logit_cap;              // > 0: every scaled score s becomes logit_cap * tanh(s / logit_cap) before the softmax
   int32_t token_band;           // 0: tokens dealt to the 8 XCDs in turn; > 0: XCD x takes tokens x*token_band .. (x+1)*token_band - 1
+  int32_t persist_workgroups;   // > 0: launches that do not split may run this many persistent workgroups (a multiple of 8) instead of one per item
   int32_t merge_in_launch;      // n_splits > 1 only.  1: the last split of a (token, head block) to arrive folds the others' partials
                                 // (needs all workgroups of a token behind one L2); 0: every split publishes, a second launch merges
 };

@@ -253,8 +253,15 @@ __device__ __forceinline__ void wait_dma(int younger_tiles) {
   else hw::wait_vmcnt<0>();
 }
 
-template <int FMT, bool CAP>
-__global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) {
+// PERSIST (launches that do not split, with several items per compute unit: prefill, dense decode
+// over many tokens): one workgroup per compute unit walks the block ids b, b + gridDim.x, ... of
+// the one-workgroup-per-item launch (gridDim.x a multiple of 8: all on its own XCD).  The next
+// item's index and Q loads go out when the current item's accumulators have been parked for the
+// epilogue, which frees the registers they land in, and its page-table look-ups follow the
+// epilogue's stores: the three dependent round trips that open an item (indices, page table,
+// first rows) shrink to the last one.
+template <int FMT, bool CAP, bool PERSIST = false>
+__global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks, int n_items) {
   // the ring area: bf16 has four whole tiles (body + RoPE block each); fp8 see Fp8Pipe
   constexpr bool kFp8 = FMT == SMLA_KV_FP8_B128;
   constexpr int kRingBytes = kFp8 ? Fp8Pipe::kRingBytes : kSlots * kTileBytes;
@@ -274,28 +281,40 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
 
   // block id -> (token, split, head block).  Ids are dealt round-robin to the 8 XCDs, so all
   // workgroups of one token (they gather overlapping rows and later merge) get ids 8 apart.
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int hb = slot % n_hblocks;
-  const int sp = (slot / n_hblocks) % p.n_splits;
-  const int t = token_of(p, xcd, slot / (n_hblocks * p.n_splits));
+  auto token_of_id = [&](int id) { return token_of(p, id & 7, (id >> 3) / (n_hblocks * p.n_splits)); };
+  auto next_item = [&](int id) {               // the next id of this workgroup that has a token (token counts are rounded up to 8 an XCD round)
+    while (id < n_items && token_of_id(id) >= p.n_tokens) id += (int)gridDim.x;
+    return id;
+  };
+  int item = PERSIST ? next_item((int)blockIdx.x) : (int)blockIdx.x;
+  if (PERSIST && item >= n_items) return;
+  int hb, sp, t, seq, head0, head;
+  bool head_ok;
+  auto place = [&](int id) {
+    const int slot = id >> 3;
+    hb = slot % n_hblocks;
+    sp = (slot / n_hblocks) % p.n_splits;
+    t = token_of_id(id);
+    seq = t / p.tokens_per_seq;
+    head0 = hb * 64 + hg * 32;
+    head = head0 + c32;
+    head_ok = head < p.n_heads;
+  };
+  place(item);
   if (t >= p.n_tokens) return;
-  const int seq = t / p.tokens_per_seq;
-  const int head0 = hb * 64 + hg * 32;
-  const int head = head0 + c32;
-  const bool head_ok = head < p.n_heads;
   const uint8_t* kv = static_cast<const uint8_t*>(p.kv);
   const int k_begin = sp * p.split_len, k_end = min(k_begin + p.split_len, p.topk);
   const WsHead ws_head = ws_read_head(p);    // read long before the split merge needs it
 
   // ---- the first chunk's index loads go out before anything else: the row list they lead to
   // (index -> page table -> row fetch) is the longest dependent chain of the kernel
-  auto load_indices = [&](int c0, int32_t (&rr)[4]) {
+  auto load_indices_of = [&](int tt, int sseq, int c0, int32_t (&rr)[4]) {
     const int c1 = min(c0 + kChunk, k_end);
     // (branch-free: with an index list every lane loads its entry, without one it loads the
     // sequence length instead; a branch per entry or per mode would make the compiler wait for
     // each load where the branches join, ahead of the Q loads that should overlap them)
     const bool listed = p.indices != nullptr;
-    const int32_t* base = listed ? p.indices + (size_t)t * p.topk : p.seq_lens + seq;
+    const int32_t* base = listed ? p.indices + (size_t)tt * p.topk : p.seq_lens + sseq;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int j = c0 + 256 * wave + 64 * k + lane;
@@ -303,6 +322,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
       rr[k] = j < c1 ? (listed ? v : (j < v ? j : -1)) : -1;
     }
   };
+  auto load_indices = [&](int c0, int32_t (&rr)[4]) { load_indices_of(t, seq, c0, rr); };
   auto translate_entries = [&](int32_t (&rr)[4]) { translate_entries4(p, seq, rr); };
   // ---- this sequence's page-table row goes global -> LDS (into the last tile body, which stays free
   // until the first chunk's row list exists) while the indices and Q are on their way, so the
@@ -330,16 +350,19 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // ---- Q^T fragments for this wavefront's 32 heads: B operand of S^T; lane holds head 16*ht + lane%16,
   // k = 32*ks + 8*(lane/16) .. +7
   bf16x8 qf[kDqk / 32][2];
+  auto load_q = [&](int tt, int hhead0) {
 #pragma unroll
-  for (int ht = 0; ht < 2; ++ht) {
-    const int hq = head0 + 16 * ht + l16;
-    // Every lane loads; a head past the end reads head 0 again (its results are never stored).
-    // Nothing touches the values here: whatever consumed them (a mask, say) would make the
-    // compiler wait for Q ahead of the row list, which only needs the index values.
-    const uint16_t* qrow = static_cast<const uint16_t*>(p.q) + ((size_t)t * p.n_heads + (hq < p.n_heads ? hq : 0)) * kDqk + 8 * q4;
+    for (int ht = 0; ht < 2; ++ht) {
+      const int hq = hhead0 + 16 * ht + l16;
+      // Every lane loads; a head past the end reads head 0 again (its results are never stored).
+      // Nothing touches the values here: whatever consumed them (a mask, say) would make the
+      // compiler wait for Q ahead of the row list, which only needs the index values.
+      const uint16_t* qrow = static_cast<const uint16_t*>(p.q) + ((size_t)tt * p.n_heads + (hq < p.n_heads ? hq : 0)) * kDqk + 8 * q4;
 #pragma unroll
-    for (int ks = 0; ks < kDqk / 32; ++ks) qf[ks][ht] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
-  }
+      for (int ks = 0; ks < kDqk / 32; ++ks) qf[ks][ht] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
+    }
+  };
+  load_q(t, head0);
   if (tid == 0) s_redo = 0;
   if (bt_in_lds) {
     // Touching the index values makes the compiler wait for exactly those loads (the Q loads
@@ -353,6 +376,15 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     translate_entries(rr_first);          // waits for the indices only; the page-table lookups overlap the Q loads
   }
 
+  // raw dot product -> base-2 exponent: one multiply, or (logit cap) the squashed score, which
+  // already is in base-2 units
+  const float sc2 = CAP ? 1.f : p.sm_scale * kLog2e;
+  [[maybe_unused]] const LogitCap cap(p.sm_scale, CAP ? p.logit_cap : 1.f);
+  const uint32_t lds_tile = hw::lds_addr(&s_ring[0]);
+  const uint32_t lds_p = hw::lds_addr(&s_p[0][0][0]);
+  const int partner = wave ^ 1;
+
+  for (;;) {       // one item a turn (a single turn unless PERSIST)
   f32x16 acc[kAccTiles];
 #pragma unroll
   for (int i = 0; i < kAccTiles; ++i)
@@ -361,13 +393,6 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   // softmax state of heads 16*ht + lane%16 (ht = 0, 1): base-2 reference (common to the pair of
   // wavefronts) and this lane's partial sum over its tokens
   float m_ref[2] = {-INFINITY, -INFINITY}, l_part[2] = {0.f, 0.f};
-  // raw dot product -> base-2 exponent: one multiply, or (logit cap) the squashed score, which
-  // already is in base-2 units
-  const float sc2 = CAP ? 1.f : p.sm_scale * kLog2e;
-  [[maybe_unused]] const LogitCap cap(p.sm_scale, CAP ? p.logit_cap : 1.f);
-  const uint32_t lds_tile = hw::lds_addr(&s_ring[0]);
-  const uint32_t lds_p = hw::lds_addr(&s_p[0][0][0]);
-  const int partner = wave ^ 1;
 
   int pass = kPassFast;
   bool first_chunk = true;
@@ -690,6 +715,19 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     for (int dt = 0; dt < kAccTiles; ++dt) stage[row * kStageStride + 32 * dt + c32_e] = acc[dt][r];
   }
   __syncthreads();                                                 // staged blocks and scalar exchange are done
+  // PERSIST: the accumulators are parked and Q has done its work, so the registers the next
+  // item's index values and Q fragments land in are free: send for them now, ahead of this
+  // item's stores.  (Nothing reads them before the stores below have been issued.)
+  [[maybe_unused]] int item_next = 0;
+  if constexpr (PERSIST) {
+    item_next = next_item(item + (int)gridDim.x);
+    if (item_next < n_items) {
+      const int slot_n = item_next >> 3, t_n = token_of_id(item_next);
+      load_indices_of(t_n, t_n / p.tokens_per_seq, k_begin, rr_first);
+      load_q(t_n, (slot_n % n_hblocks) * 64 + hg * 32);
+      if (tid_e == 0) s_redo = 0;
+    }
+  }
   if (g_e == 0) s_x[wave][c32_e] = inv;                                // per-row normaliser
   hw::wave_lds_order();
   const int n_rows = max(0, min(32, p.n_heads - head0));           // head rows that exist (wave-uniform; 0: the whole head group lies past the last head)
@@ -701,7 +739,7 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
     w.y = pack_bf16(v.z, v.w);
     *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + ((size_t)t * p.n_heads + head0 + row) * kDv + col4) = w;
   };
-  if (p.n_splits == 1) {
+  if (PERSIST || p.n_splits == 1) {
     if (dh == 0 && g_e == 0 && head_ok_e) p.lse[(size_t)t * p.n_heads + head_e] = lse_nat;
     for (int row = 0; row < n_rows; ++row) {
       const float sc = s_x[wave][row];
@@ -709,7 +747,15 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
       v.x *= sc; v.y *= sc; v.z *= sc; v.w *= sc;
       store_bf16x4(row, v);
     }
-    return;
+    if constexpr (PERSIST) {
+      if (item_next >= n_items) return;
+      item = item_next;
+      place(item);                           // from here on t, seq, head0 ... are the next item's
+      translate_entries(rr_first);           // waits for its index values only; page-table look-ups straight from memory
+      continue;                              // (the barrier that opens its first chunk also ends everyone's reads of the parked blocks)
+    } else {
+      return;
+    }
   }
 
   // ---- split merge inside the launch.  Every (token, head block) owns one 64-bit word:
@@ -817,6 +863,8 @@ __global__ __launch_bounds__(kNT) void fwd_tall_kernel(Params p, int n_hblocks) 
   }
   __syncthreads();
   if (tid_e == 0) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+  return;
+  }      // (the loop over items)
 }
 
 template <int FMT, bool CAP>
@@ -824,7 +872,19 @@ static int launch_tall_impl(const Params& p, hipStream_t s) {
   const int n_hblocks = (p.n_heads + 63) / 64;
   const long long blocks = ((long long)p.n_tokens + 7) / 8 * 8 * n_hblocks * p.n_splits;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_tall_kernel<FMT, CAP>), dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
+  // Persistent workgroups where a compute unit has several items to go through and nothing is
+  // split (FLAGTREE_SMLA_PERSIST=1, opt-in until measured): one workgroup per compute unit; the
+  // count must be a multiple of 8 for the ids a workgroup walks to stay on its XCD.
+  // (built for bf16 rows without a logit cap, the prefill and dense-decode case; the other
+  // instantiations have no registers to spare for the loop-carried state)
+  if constexpr (FMT == SMLA_KV_BF16 && !CAP) {
+    if (p.persist_workgroups > 0 && p.n_splits == 1 && blocks >= 2LL * p.persist_workgroups) {
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_tall_kernel<FMT, CAP, true>), dim3((unsigned)p.persist_workgroups), dim3(kNT), 0, s, p, n_hblocks,
+                         (int)blocks);
+      return hip_status(hipGetLastError());
+    }
+  }
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_tall_kernel<FMT, CAP>), dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks, (int)blocks);
   return hip_status(hipGetLastError());
 }
 

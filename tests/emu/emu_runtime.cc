@@ -115,6 +115,7 @@ unsigned g_wave_skew = 0;
 unsigned g_concurrent = 0;         // 0 / 1: workgroups run one after the other; n: up to n share the machine
 unsigned g_concurrent_seed = 0;
 unsigned long long g_launches = 0;
+unsigned long long g_blocks = 0;
 unsigned long long g_polls = 0;
 int g_cu_count = 256;
 std::vector<char*> g_stacks;
@@ -519,6 +520,7 @@ void launch(Dim3 grid, Dim3 block, const std::function<void()>& body) {
   g_grid_dim = grid;
   g_body = &body;
   const size_t n_blocks = (size_t)grid.x * grid.y * grid.z;
+  g_blocks += n_blocks;
   std::vector<size_t> order(n_blocks);
   for (size_t i = 0; i < n_blocks; ++i) order[i] = i;
   if (g_order_seed) {
@@ -543,6 +545,7 @@ void emu_set_block_order(unsigned seed) { emu::g_order_seed = seed; }
 void emu_set_wave_skew(unsigned seed) { emu::g_wave_skew = seed; }
 void emu_set_concurrent_blocks(unsigned n, unsigned seed) { emu::g_concurrent = n; emu::g_concurrent_seed = seed; }
 unsigned long long emu_launch_count(void) { return emu::g_launches; }
+unsigned long long emu_block_count(void) { return emu::g_blocks; }
 unsigned long long emu_poll_count(void) { return emu::g_polls; }
 void emu_set_cu_count(int n) { emu::g_cu_count = n; }
 void emu_set_lds_profile(int on) {

@@ -86,6 +86,7 @@ void emu_set_wave_skew(unsigned seed);   // 0: a workgroup's wavefronts advance 
 // (a workgroup that polls for another one's writes then really waits); else one workgroup after the other
 void emu_set_concurrent_blocks(unsigned n, unsigned seed);
 unsigned long long emu_launch_count(void);
+unsigned long long emu_block_count(void);  // workgroups of all launches since the library was loaded
 unsigned long long emu_poll_count(void);  // times a lane gave way inside a polling loop since the library was loaded
 void emu_set_cu_count(int n);            // before the library's first query (it caches the answer); default 256
 void emu_set_lds_profile(int on);        // 1: count bank passes of the kernels' addressed LDS accesses (slower); resets the counts

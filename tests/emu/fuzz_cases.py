@@ -25,7 +25,7 @@ from _util import max_abs, oracle_inputs, to_np   # noqa: E402
 
 G = harness.Guarded
 SWITCHES = ("FLAGTREE_SMLA_FEW_FP8", "FLAGTREE_SMLA_FP8_MFMA", "FLAGTREE_SMLA_HEAD_GROUPS", "FLAGTREE_SMLA_TOKEN_BANDS",
-            "FLAGTREE_SMLA_SEPARATE_MERGE")
+            "FLAGTREE_SMLA_SEPARATE_MERGE", "FLAGTREE_SMLA_PERSIST")
 
 
 def random_schedule(rng):
@@ -60,6 +60,8 @@ def forward_case(seed):
         os.environ["FLAGTREE_SMLA_TOKEN_BANDS"] = "1"
     if rng.random() < 0.25:
         os.environ["FLAGTREE_SMLA_SEPARATE_MERGE"] = "1"
+    if rng.random() < 0.5:
+        os.environ["FLAGTREE_SMLA_PERSIST"] = "1"           # (takes effect on unsplit many-heads launches with enough items)
     cap = float(rng.choice([0.0, 0.0, 0.05])) if dense else 0.0
     if paged:
         pps = -(-ctx // page_size)

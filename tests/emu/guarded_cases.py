@@ -29,7 +29,7 @@ def _guard_cfg(cfg, end):
 
 def forward_case(make, n_splits, dense=False, env=None):
     def run(end):
-        for k in ("FLAGTREE_SMLA_FEW_FP8", "FLAGTREE_SMLA_HEAD_GROUPS", "FLAGTREE_SMLA_FP8_MFMA"):
+        for k in ("FLAGTREE_SMLA_FEW_FP8", "FLAGTREE_SMLA_HEAD_GROUPS", "FLAGTREE_SMLA_FP8_MFMA", "FLAGTREE_SMLA_PERSIST"):
             os.environ.pop(k, None)
         os.environ.update(env or {})
         cfg = make()
@@ -172,6 +172,8 @@ CASES = {
     "fp8_mfma_split": forward_case(lambda: fp8_cfg(2, 16, 4, 150), 2, env={"FLAGTREE_SMLA_FP8_MFMA": "1"}),
     "fp8_mfma_ragged_heads": forward_case(lambda: fp8_cfg(1, 9, 4, 100), 1, env={"FLAGTREE_SMLA_FP8_MFMA": "1"}),
     "fp8_mfma_short_lists": forward_case(lambda: fp8_cfg(3, 30, 2, 40), 1, env={"FLAGTREE_SMLA_FP8_MFMA": "1"}),
+    "tall_bf16_persistent": forward_case(lambda: workloads.prefill_causal_bf16("cpu", tokens=43, heads=72, topk=48), 1,
+                                         env={"FLAGTREE_SMLA_PERSIST": "1"}),
     "dense_tall": forward_case(lambda: workloads.decode_bf16("cpu", batch=3, heads=128, pages_per_seq=3, topk=64), 2, dense=True),
     "dense_short_fp8": forward_case(lambda: fp8_cfg(3, 16, 3, 64), 1, dense=True),
     "scalar_f32": forward_case(lambda: workloads.plumbing_f32("cpu", tokens=2, heads=16, s_kv=256, topk=40), 1),

@@ -36,6 +36,7 @@ def lib():
         l.emu_set_wave_skew.argtypes = [ctypes.c_uint]
         l.emu_set_concurrent_blocks.argtypes = [ctypes.c_uint, ctypes.c_uint]
         l.emu_launch_count.restype = ctypes.c_ulonglong
+        l.emu_block_count.restype = ctypes.c_ulonglong
         l.emu_poll_count.restype = ctypes.c_ulonglong
         l.emu_set_cu_count.argtypes = [ctypes.c_int]
         l.emu_set_lds_profile.argtypes = [ctypes.c_int]

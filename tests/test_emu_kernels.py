@@ -322,6 +322,48 @@ def test_column_split_kernel_edge_cases_redo_and_dense(few_fp8_kernel):
         assert max_abs(to_np(lse), wl) <= LSE_TOL and max_abs(to_np(out), wo) <= OUT_TOL
 
 
+@pytest.mark.parametrize("case", ["prefill", "prefill_200_heads_two_chunks", "decode_many_tokens", "dense"])
+def test_persistent_workgroups_give_the_same_bits(case, monkeypatch):
+    """FLAGTREE_SMLA_PERSIST=1: launches of the many-heads kernel that do not split and have at least
+    two items per compute unit run one workgroup per compute unit (16 here), which walks its items
+    and sends for the next one's indices and Q while the current one's output is on its way out.
+    Every item is computed by the same code on the same data: the same bits as one workgroup per
+    item, with wavefronts in step, skewed, with moves landing at issue, and with workgroups
+    sharing the machine."""
+    from flagtree_amd import workloads
+    lens = None
+    if case == "prefill":
+        cfg = workloads.prefill_causal_bf16("cpu", tokens=43, heads=128, topk=48)          # 43 tokens: ids without a token in between
+    elif case == "prefill_200_heads_two_chunks":
+        cfg = workloads.prefill_causal_bf16("cpu", tokens=40, heads=200, topk=1100)
+    elif case == "decode_many_tokens":
+        cfg = workloads.decode_bf16("cpu", batch=37, heads=128, pages_per_seq=8, topk=130, pad_frac=0.1)
+    else:
+        cfg = workloads.decode_bf16("cpu", batch=33, heads=128, pages_per_seq=3, topk=64)
+        lens = torch.randint(0, 3 * 64 + 1, (33,), generator=torch.Generator().manual_seed(2), dtype=torch.int32)
+    lib = harness.lib()
+    monkeypatch.delenv("FLAGTREE_SMLA_PERSIST", raising=False)
+    blocks = lib.emu_block_count()
+    out0, lse0, rc = harness.forward(cfg, n_splits=1, dense_lens=lens)
+    one_per_item = lib.emu_block_count() - blocks
+    assert rc == 0 and one_per_item >= 2 * harness.EMU_CUS
+    monkeypatch.setenv("FLAGTREE_SMLA_PERSIST", "1")
+    for skew, eager, together in ((0, False, 0), (3, True, 0), (5, False, 4)):
+        harness.configure(wave_skew_seed=skew, dma_eager=eager, concurrent_blocks=together, concurrent_seed=3)
+        blocks = lib.emu_block_count()
+        out1, lse1, rc = harness.forward(cfg, n_splits=1, dense_lens=lens)
+        assert rc == 0 and lib.emu_block_count() - blocks == harness.EMU_CUS          # it is the persistent launch
+        assert torch.equal(out0.view(torch.int16), out1.view(torch.int16)) and torch.equal(lse0, lse1), (skew, eager, together)
+    harness.configure()
+    if lens is None:
+        _check(cfg, out1, lse1)
+    # a split launch, or one with fewer than two items per compute unit, is left alone
+    blocks = lib.emu_block_count()
+    small = workloads.decode_bf16("cpu", batch=3, heads=128, pages_per_seq=8, topk=130, pad_frac=0.1)
+    harness.forward(small, n_splits=1)
+    assert lib.emu_block_count() - blocks == 8 * 2
+
+
 def test_more_than_one_chunk_of_the_list():
     """Lists longer than the 1024 entries the kernels compact at a time, ragged last tile."""
     from flagtree_amd import workloads

@@ -219,3 +219,38 @@ def test_token_bands_give_the_same_bits(dev, monkeypatch, heads, n_splits, token
     out1, lse1 = _fwd(cfg, n_splits=n_splits)
     assert torch.equal(out0.view(torch.int16), out1.view(torch.int16)) and torch.equal(lse0, lse1)
     _check(cfg, out1, lse1)
+
+
+# ---- persistent workgroups for unsplit many-heads launches (opt-in) ------------------------------
+
+@pytest.mark.parametrize("case", ["prefill", "dense"])
+def test_persistent_workgroups_give_the_same_bits(dev, monkeypatch, case):
+    """FLAGTREE_SMLA_PERSIST=1: one workgroup per compute unit walks its (token, head block) items and
+    sends for the next item's indices and Q under the current item's output stores.  Same code on
+    the same data per item: the same bits as one workgroup per item."""
+    import flagtree_amd as ft
+    from flagtree_amd import workloads
+    monkeypatch.delenv("FLAGTREE_SMLA_PERSIST", raising=False)
+    if case == "prefill":
+        cfg = workloads.prefill_causal_bf16(dev, tokens=700, heads=128, topk=256)          # 1408 items on 256 compute units
+        out0, lse0 = _fwd(cfg, n_splits=1)
+        monkeypatch.setenv("FLAGTREE_SMLA_PERSIST", "1")
+        out1, lse1 = _fwd(cfg, n_splits=1)
+        torch.cuda.synchronize()
+        rows = slice(300, 340)
+        sub = dict(cfg, q=cfg["q"][:, rows], indices=cfg["indices"][:, rows])
+        ro, rl = run_oracle(sub)
+        assert max_abs(to_np(out1[:, rows]).reshape(ro.shape), ro) <= OUT_TOL and max_abs(to_np(lse1[:, rows]).reshape(rl.shape), rl) <= LSE_TOL
+    else:
+        B, L, page_size = 300, 400, 64
+        g = torch.Generator().manual_seed(21)
+        n_pages = -(-L // page_size)
+        req = torch.randperm(B * n_pages, generator=g).to(torch.int32).view(B, n_pages).to(dev)
+        lens = torch.randint(1, L + 1, (B,), generator=g, dtype=torch.int32).to(dev)
+        k_buffer = (torch.randn((B * n_pages * page_size, 576), generator=g) * 0.1).to(torch.bfloat16).to(dev).view(-1, page_size, 576)
+        q = (torch.randn((B, 128, 576), generator=g) * 0.1).to(torch.bfloat16).to(dev)
+        out0, lse0 = ft.decode_attention_fwd(q, k_buffer, None, None, req, lens, None, 1, 576 ** -0.5, page_size)
+        monkeypatch.setenv("FLAGTREE_SMLA_PERSIST", "1")
+        out1, lse1 = ft.decode_attention_fwd(q, k_buffer, None, None, req, lens, None, 1, 576 ** -0.5, page_size)
+        torch.cuda.synchronize()
+    assert torch.equal(out0, out1) and torch.equal(lse0, lse1)
