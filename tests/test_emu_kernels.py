@@ -969,7 +969,7 @@ def test_local_gemm(m, n, k, chunks):
 @pytest.mark.parametrize("m,n,k,chunks", [(2048, 1280, 128, 2),     # 40 tiles on 16 units: two whole tiles chained per workgroup, then a half tile
                                           (2048, 1280, 192, 8),     # three K-steps: the buffers swap roles from tile to tile
                                           (2048, 1024, 64, 1),      # one K-step a tile, 32 tiles: two chained whole tiles, no halves
-                                          (4096, 1536, 128, 4),     # 96 tiles: six chained whole tiles per workgroup
+                                          (2048, 2048, 64, 4),      # 64 tiles: four chained whole tiles per workgroup
                                           (2048, 768, 128, 2)])     # 24 tiles: one whole tile and one half tile per workgroup
 def test_local_gemm_by_persistent_workgroups(m, n, k, chunks, monkeypatch):
     """FLAGTREE_SMLA_GEMM_CHAIN=1: one workgroup per compute unit walks its tiles; the next tile's
