@@ -223,55 +223,73 @@ def main():
                                  block_table=c["block_table"], page_size=c["page_size"], kv_format=fmt,
                                  n_splits=n_splits, workspace=ws)
 
-    for i in range(a.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    # The forward is a single kernel launch (the split merge happens inside it; on a device whose
-    # XCD layout the library does not know, a merge launch follows it), issued on torch's current
-    # stream.  One HIP event pair on that stream brackets the K launches: the
-    # span divided by K is the average launch duration including the gap between back-to-back
-    # launches; a second pass with one event pair per launch gives the per-launch distribution.
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(a.steps):
-        step(i)
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / a.steps
-    kern_ms = e0.elapsed_time(e1) / a.steps
-    n_dist = min(a.steps, 50)
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_dist)]
-    for i in range(n_dist):
-        ev[i][0].record()
-        step(i)
-        ev[i][1].record()
-    torch.cuda.synchronize()
-    op_ms = sorted(x.elapsed_time(y) for x, y in ev)
-    op_ms_avg = sum(op_ms) / len(op_ms)
-    tail_ms = None
-    if tail_sets:
-        for i in range(min(a.warmup, 10)):
-            step(i, tail_sets)
+    def run_timed():
+        for i in range(a.warmup):
+            step(i)
         torch.cuda.synchronize()
-        f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        f0.record()
+        # The forward is a single kernel launch (the split merge happens inside it; on a device whose
+        # XCD layout the library does not know, a merge launch follows it), issued on torch's current
+        # stream.  One HIP event pair on that stream brackets the K launches: the
+        # span divided by K is the average launch duration including the gap between back-to-back
+        # launches; a second pass with one event pair per launch gives the per-launch distribution.
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
         for i in range(a.steps):
-            step(i, tail_sets)
-        f1.record()
+            step(i)
+        e1.record()
         torch.cuda.synchronize()
-        tail_ms = f0.elapsed_time(f1) / a.steps
-    # A split merge that gave up marks its rows with a NaN LSE and flags the workspace, and every
-    # later launch on that workspace gives up too: no figure is printed for such a run.
-    if ws is not None:
-        ft.workspace_status(ws)                       # raises when any launch above flagged it
-    last_lse = step(0)[1]
-    torch.cuda.synchronize()
-    if not bool(torch.isfinite(last_lse).all().item()):
-        raise RuntimeError("non-finite LSE after the timed loop: the run measured a launch that did not compute")
-    if ws is not None:
-        ft.workspace_status(ws)
+        wall = time.perf_counter() - t0
+        ms_per_step = wall * 1e3 / a.steps
+        kern_ms = e0.elapsed_time(e1) / a.steps
+        n_dist = min(a.steps, 50)
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_dist)]
+        for i in range(n_dist):
+            ev[i][0].record()
+            step(i)
+            ev[i][1].record()
+        torch.cuda.synchronize()
+        op_ms = sorted(x.elapsed_time(y) for x, y in ev)
+        op_ms_avg = sum(op_ms) / len(op_ms)
+        tail_ms = None
+        if tail_sets:
+            for i in range(min(a.warmup, 10)):
+                step(i, tail_sets)
+            torch.cuda.synchronize()
+            f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            f0.record()
+            for i in range(a.steps):
+                step(i, tail_sets)
+            f1.record()
+            torch.cuda.synchronize()
+            tail_ms = f0.elapsed_time(f1) / a.steps
+        # A split merge that gave up marks its rows with a NaN LSE and flags the workspace, and every
+        # later launch on that workspace gives up too: no figure is printed for such a run.
+        if ws is not None:
+            ft.workspace_status(ws)                       # raises when any launch above flagged it
+        last_lse = step(0)[1]
+        torch.cuda.synchronize()
+        if not bool(torch.isfinite(last_lse).all().item()):
+            raise RuntimeError("non-finite LSE after the timed loop: the run measured a launch that did not compute")
+        if ws is not None:
+            ft.workspace_status(ws)
+
+        return ms_per_step, kern_ms, op_ms, op_ms_avg, tail_ms
+
+    # A merge inside the launch that gives up (a workspace flagged, NaN rows) means this device does
+    # not do what the in-launch merge relies on.  The run is then repeated once with the merge as a
+    # second launch, which relies on nothing but the kernel boundary, and the line says so.
+    merge_note = None
+    try:
+        ms_per_step, kern_ms, op_ms, op_ms_avg, tail_ms = run_timed()
+    except RuntimeError as e:
+        if ws is None or os.environ.get("FLAGTREE_SMLA_SEPARATE_MERGE") == "1":
+            raise
+        merge_note = f"second launch (the merge inside the launch failed on this device: {e})"
+        print("bench.py: " + merge_note, file=sys.stderr)
+        os.environ["FLAGTREE_SMLA_SEPARATE_MERGE"] = "1"
+        ws = ft.make_workspace(ws_bytes, dev)
+        ms_per_step, kern_ms, op_ms, op_ms_avg, tail_ms = run_timed()
 
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     gbs = nbytes / (ms_per_step * 1e-3) / 1e9
@@ -315,6 +333,8 @@ def main():
         "roofline": roof,
         "timing": TIMING_NOTE,
     }
+    res["config"]["split_merge"] = ("none" if n_splits == 1 else merge_note if merge_note else
+                                    "inside the launch" if lib.smla_merge_in_launch() else "second launch")
     if tail_ms is not None:
         res["padding_order"] = {"shuffled_kernel_ms": kern_ms, "tail_kernel_ms": tail_ms,
                                 "note": "same index sets, -1 entries spread through the list (the headline) / moved to its end"}
