@@ -321,7 +321,7 @@ def main():
             "prefill_causal_bf16": "causal prefill S=8192 h=128 topk=2048"}[a.workload],
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "fp8_e4m3" if (a.fp8_mfma and hbm_bound) else "bf16", "data": "synthetic",
         "config": {"workload": a.workload, "batch": cfg["q"].shape[0], "heads": H, "topk": K,
                    "n_valid": n_valid, "kv_format": fmt, "page_size": cfg["page_size"],
                    "n_splits": n_splits, "input_sets": len(sets), "token_bands": bool(a.token_bands),
