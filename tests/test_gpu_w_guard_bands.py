@@ -1,9 +1,5 @@
 """GPU check that no entry point writes outside the buffers it is given.
 
-Not collected yet (the file name does not start with ``test_``): it was written when no GPU was
-available and has not run.  Run it by naming the file; rename it to ``test_zz_guard_bands.py``
-once it passes.
-
 Every output lives in the middle of a larger buffer filled with a byte pattern, 64 KB of it on
 either side; after the call through the C ABI the pattern must be intact and the output must be
 bit-identical to what the Python wrapper (whose results the parity tests check) returns for the
