@@ -214,8 +214,12 @@ __device__ __forceinline__ void tile_accumulate(uint32_t tile, const bf16x8 (&pa
   __builtin_amdgcn_sched_barrier(0);
 }
 
-template <int FMT, bool CAP>
-__global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks) {
+// PERSIST: as in fwd_tall_kernel -- for launches that do not split and have several items per
+// compute unit, one workgroup per compute unit walks the block ids b, b + gridDim.x, ... of the
+// one-workgroup-per-item launch and sends for the next item's indices and Q at the top of the
+// current item's epilogue, when Q has done its work and the registers are free.
+template <int FMT, bool CAP, bool PERSIST = false>
+__global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks, int n_items) {
   // the ring area: bf16 has four whole tiles (body + RoPE block each); fp8 see smla_fp8_pipe.h
   constexpr bool kFp8 = FMT == SMLA_KV_FP8_B128;
   static_assert(Fp8Pipe::kRingBytes <= kSlots * kTileBytes, "the fp8 carving fits the same area");
@@ -232,23 +236,34 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   const int l16 = lane & 15, q4 = lane >> 4;
 
   // block id -> (token, split, head block); all workgroups of a token get ids 8 apart (one XCD)
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int hb = slot % n_hblocks;
-  const int sp = (slot / n_hblocks) % p.n_splits;
-  const int t = token_of(p, xcd, slot / (n_hblocks * p.n_splits));
+  auto token_of_id = [&](int id) { return token_of(p, id & 7, (id >> 3) / (n_hblocks * p.n_splits)); };
+  auto next_item = [&](int id) {               // the next id of this workgroup that has a token
+    while (id < n_items && token_of_id(id) >= p.n_tokens) id += (int)gridDim.x;
+    return id;
+  };
+  int item = PERSIST ? next_item((int)blockIdx.x) : (int)blockIdx.x;
+  if (PERSIST && item >= n_items) return;
+  int hb, sp, t, seq, head0;                                      // head0: first head of this wavefront
+  auto place = [&](int id) {
+    const int slot = id >> 3;
+    hb = slot % n_hblocks;
+    sp = (slot / n_hblocks) % p.n_splits;
+    t = token_of_id(id);
+    seq = t / p.tokens_per_seq;
+    head0 = hb * 128 + wave * 32;
+  };
+  place(item);
   if (t >= p.n_tokens) return;
-  const int seq = t / p.tokens_per_seq;
-  const int head0 = hb * 128 + wave * 32;                         // first head of this wavefront
   const uint8_t* kv = static_cast<const uint8_t*>(p.kv);
   const int k_begin = sp * p.split_len, k_end = min(k_begin + p.split_len, p.topk);
   const WsHead ws_head = ws_read_head(p);    // read long before the split merge needs it
 
   // ---- the first chunk's index loads go out before anything else: the row list they lead to
   // (index -> page table -> row fetch) is the longest dependent chain of the kernel
-  auto load_indices = [&](int c0, int32_t (&rr)[4]) {
+  auto load_indices_of = [&](int tt, int sseq, int c0, int32_t (&rr)[4]) {
     const int c1 = min(c0 + kChunk, k_end);
     const bool listed = p.indices != nullptr;
-    const int32_t* base = listed ? p.indices + (size_t)t * p.topk : p.seq_lens + seq;
+    const int32_t* base = listed ? p.indices + (size_t)tt * p.topk : p.seq_lens + sseq;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int j = c0 + 256 * wave + 64 * k + lane;
@@ -256,6 +271,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
       rr[k] = j < c1 ? (listed ? v : (j < v ? j : -1)) : -1;
     }
   };
+  auto load_indices = [&](int c0, int32_t (&rr)[4]) { load_indices_of(t, seq, c0, rr); };
   // the sequence's page-table row goes global -> LDS (last tile body, free until the first chunk's
   // row list exists), issued ahead of the index loads so that it has landed once they have
   const int32_t* bt_row = p.block_table ? p.block_table + (size_t)seq * p.bt_stride : nullptr;
@@ -278,13 +294,16 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   // stored); nothing touches the values here, so the compiler does not wait for Q ahead of the
   // row list.
   bf16x8 qf[kDqk / 32][2];
+  auto load_q = [&](int tt, int hhead0) {
 #pragma unroll
-  for (int ht = 0; ht < 2; ++ht) {
-    const int hq = head0 + 16 * ht + l16;
-    const uint16_t* qrow = static_cast<const uint16_t*>(p.q) + ((size_t)t * p.n_heads + (hq < p.n_heads ? hq : 0)) * kDqk + 8 * q4;
+    for (int ht = 0; ht < 2; ++ht) {
+      const int hq = hhead0 + 16 * ht + l16;
+      const uint16_t* qrow = static_cast<const uint16_t*>(p.q) + ((size_t)tt * p.n_heads + (hq < p.n_heads ? hq : 0)) * kDqk + 8 * q4;
 #pragma unroll
-    for (int ks = 0; ks < kDqk / 32; ++ks) qf[ks][ht] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
-  }
+      for (int ks = 0; ks < kDqk / 32; ++ks) qf[ks][ht] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
+    }
+  };
+  load_q(t, head0);
   if (tid == 0) s_redo = 0;
   if (bt_in_lds) {
     hw::wait_for_loads_of(rr_first[0], rr_first[1], rr_first[2], rr_first[3]);
@@ -296,6 +315,10 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
     translate_entries4(p, seq, rr_first);
   }
 
+  const float sc2 = CAP ? 1.f : p.sm_scale * kLog2e;
+  [[maybe_unused]] const LogitCap cap(p.sm_scale, CAP ? p.logit_cap : 1.f);
+
+  for (;;) {       // one item a turn (a single turn unless PERSIST)
   f32x4 acc[2][kColTiles];
 #pragma unroll
   for (int ht = 0; ht < 2; ++ht)
@@ -303,8 +326,6 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
     for (int ct = 0; ct < kColTiles; ++ct) acc[ht][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   // softmax state of heads 16 ht + l16: base-2 reference and this lane's partial row sum (its 8 tokens of every tile)
   float m_ref[2] = {-INFINITY, -INFINITY}, l_part[2] = {0.f, 0.f};
-  const float sc2 = CAP ? 1.f : p.sm_scale * kLog2e;
-  [[maybe_unused]] const LogitCap cap(p.sm_scale, CAP ? p.logit_cap : 1.f);
 
   int pass = kPassFast;
   bool first_chunk = true;
@@ -584,6 +605,18 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   // LDS 16 head rows (one head tile) at a time: parked as accumulator tiles (lane = column, register
   // = row), read back one head row at a time, 8 consecutive columns per lane.
   __syncthreads();                           // the ring is free
+  // PERSIST: Q has done its work and the first chunk's index values theirs; the registers they
+  // live in take the next item's, sent for now, ahead of this item's stores.
+  [[maybe_unused]] int item_next = 0;
+  if constexpr (PERSIST) {
+    item_next = next_item(item + (int)gridDim.x);
+    if (item_next < n_items) {
+      const int slot_n = item_next >> 3, t_n = token_of_id(item_next);
+      load_indices_of(t_n, t_n / p.tokens_per_seq, k_begin, rr_first);
+      load_q(t_n, (slot_n % n_hblocks) * 128 + wave * 32);
+      if (tid == 0) s_redo = 0;
+    }
+  }
   if (p.n_splits > 1 && tid == 0)
     s_nvalid = ws_arrive(p, p.counters + (size_t)t * n_hblocks + hb, ws_head, p.n_splits, sp);
   const int lane_e = hw::lane_id();          // (lane coordinates retaken here rather than carried through the loop)
@@ -631,7 +664,7 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   auto head_ok = [&](int ht) { return head0 + 16 * ht + l16_e < p.n_heads; };
 
   const int ns = p.n_splits;
-  if (ns == 1) {
+  if (PERSIST || ns == 1) {
 #pragma unroll
     for (int ht = 0; ht < 2; ++ht) {
       if (q4_e == 0 && head_ok(ht)) p.lse[lse_index(ht)] = lse_nat[ht];
@@ -639,7 +672,15 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
       for (int row = 0; row < 16; ++row)
         if (16 * ht + row < n_rows) store_bf16x8(16 * ht + row, staged(row, 0), staged(row, 1));
     }
-    return;
+    if constexpr (PERSIST) {
+      if (item_next >= n_items) return;
+      item = item_next;
+      place(item);                           // from here on t, seq, head0 are the next item's
+      translate_entries4(p, seq, rr_first);  // waits for its index values only; page-table look-ups straight from memory
+      continue;                              // (the barrier that opens its first chunk also ends everyone's reads of the staged rows)
+    } else {
+      return;
+    }
   }
 
   // ---- split merge inside the launch (protocol and failure handling: ws_arrive / ws_wait_published
@@ -765,6 +806,8 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks)
   }
   __syncthreads();
   if (wave == 0 && lane_e == 0) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+  return;
+  }      // (the loop over items)
 }
 
 template <int FMT, bool CAP>
@@ -772,7 +815,15 @@ int launch_impl(const Params& p, hipStream_t s) {
   const int n_hblocks = (p.n_heads + 127) / 128;
   const long long blocks = ((long long)p.n_tokens + 7) / 8 * 8 * n_hblocks * p.n_splits;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_group_kernel<FMT, CAP>), dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks);
+  // persistent workgroups (see fwd_tall_kernel's launcher): bf16 rows without a logit cap
+  if constexpr (FMT == SMLA_KV_BF16 && !CAP) {
+    if (p.persist_workgroups > 0 && p.n_splits == 1 && blocks >= 2LL * p.persist_workgroups) {
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_group_kernel<FMT, CAP, true>), dim3((unsigned)p.persist_workgroups), dim3(kNT), 0, s, p,
+                         n_hblocks, (int)blocks);
+      return hip_status(hipGetLastError());
+    }
+  }
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(fwd_group_kernel<FMT, CAP>), dim3((unsigned)blocks), dim3(kNT), 0, s, p, n_hblocks, (int)blocks);
   return hip_status(hipGetLastError());
 }
 

@@ -322,8 +322,9 @@ def test_column_split_kernel_edge_cases_redo_and_dense(few_fp8_kernel):
         assert max_abs(to_np(lse), wl) <= LSE_TOL and max_abs(to_np(out), wo) <= OUT_TOL
 
 
+@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group"])
 @pytest.mark.parametrize("case", ["prefill", "prefill_200_heads_two_chunks", "decode_many_tokens", "dense"])
-def test_persistent_workgroups_give_the_same_bits(case, monkeypatch):
+def test_persistent_workgroups_give_the_same_bits(case, kernel, monkeypatch):
     """FLAGTREE_SMLA_PERSIST=1: launches of the many-heads kernel that do not split and have at least
     two items per compute unit run one workgroup per compute unit (16 here), which walks its items
     and sends for the next one's indices and Q while the current one's output is on its way out.
@@ -343,6 +344,9 @@ def test_persistent_workgroups_give_the_same_bits(case, monkeypatch):
         lens = torch.randint(0, 3 * 64 + 1, (33,), generator=torch.Generator().manual_seed(2), dtype=torch.int32)
     lib = harness.lib()
     monkeypatch.delenv("FLAGTREE_SMLA_PERSIST", raising=False)
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel == "wavefront_per_head_group" else "0")
+    if kernel == "wavefront_per_head_group" and case == "dense":
+        cfg = workloads.decode_bf16("cpu", batch=33, heads=200, pages_per_seq=3, topk=64)       # 128 heads a workgroup: two head blocks an item
     blocks = lib.emu_block_count()
     out0, lse0, rc = harness.forward(cfg, n_splits=1, dense_lens=lens)
     one_per_item = lib.emu_block_count() - blocks
@@ -361,7 +365,7 @@ def test_persistent_workgroups_give_the_same_bits(case, monkeypatch):
     blocks = lib.emu_block_count()
     small = workloads.decode_bf16("cpu", batch=3, heads=128, pages_per_seq=8, topk=130, pad_frac=0.1)
     harness.forward(small, n_splits=1)
-    assert lib.emu_block_count() - blocks == 8 * 2
+    assert lib.emu_block_count() - blocks == 8 * (2 if kernel == "many_heads" else 1)
 
 
 def test_more_than_one_chunk_of_the_list():

@@ -223,16 +223,18 @@ def test_token_bands_give_the_same_bits(dev, monkeypatch, heads, n_splits, token
 
 # ---- persistent workgroups for unsplit many-heads launches (opt-in) ------------------------------
 
+@pytest.mark.parametrize("kernel", ["many_heads", "wavefront_per_head_group"])
 @pytest.mark.parametrize("case", ["prefill", "dense"])
-def test_persistent_workgroups_give_the_same_bits(dev, monkeypatch, case):
+def test_persistent_workgroups_give_the_same_bits(dev, monkeypatch, case, kernel):
     """FLAGTREE_SMLA_PERSIST=1: one workgroup per compute unit walks its (token, head block) items and
     sends for the next item's indices and Q under the current item's output stores.  Same code on
     the same data per item: the same bits as one workgroup per item."""
     import flagtree_amd as ft
     from flagtree_amd import workloads
     monkeypatch.delenv("FLAGTREE_SMLA_PERSIST", raising=False)
+    monkeypatch.setenv("FLAGTREE_SMLA_HEAD_GROUPS", "1" if kernel == "wavefront_per_head_group" else "0")
     if case == "prefill":
-        cfg = workloads.prefill_causal_bf16(dev, tokens=700, heads=128, topk=256)          # 1408 items on 256 compute units
+        cfg = workloads.prefill_causal_bf16(dev, tokens=700, heads=128, topk=256)          # 1408 (or 704) items on 256 compute units
         out0, lse0 = _fwd(cfg, n_splits=1)
         monkeypatch.setenv("FLAGTREE_SMLA_PERSIST", "1")
         out1, lse1 = _fwd(cfg, n_splits=1)
@@ -242,7 +244,7 @@ def test_persistent_workgroups_give_the_same_bits(dev, monkeypatch, case):
         ro, rl = run_oracle(sub)
         assert max_abs(to_np(out1[:, rows]).reshape(ro.shape), ro) <= OUT_TOL and max_abs(to_np(lse1[:, rows]).reshape(rl.shape), rl) <= LSE_TOL
     else:
-        B, L, page_size = 300, 400, 64
+        B, L, page_size = 600, 400, 64
         g = torch.Generator().manual_seed(21)
         n_pages = -(-L // page_size)
         req = torch.randperm(B * n_pages, generator=g).to(torch.int32).view(B, n_pages).to(dev)
