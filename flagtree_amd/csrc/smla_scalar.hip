@@ -226,8 +226,27 @@ int launch_merge(const float* part_out, const float* part_lse, void* out, float*
 // bits of the fp32 mantissa (three mantissa bits kept, the fourth set, nothing below).  Lanes
 // with a product within 5 units of that pattern, or with a value small enough for an fp8
 // subnormal (other midpoints), divide.
+// a 64-bit value that every lane of the wavefront holds alike, moved to scalar registers
+__device__ __forceinline__ int64_t wave_uniform(int64_t v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 constexpr int kRowsPerWave = 4;                    // rows a wavefront has in flight: one row a wavefront leaves the
                                                    // memory pipe half empty (36 KB of loads per CU against ~64 KB of latency x bandwidth)
+
+// x / 448 correctly rounded, for x >= 2^-126 * 448 and finite, in three operations instead of the
+// dozen of an IEEE division: q0 = x * RN(1/448) is within a unit of the quotient, the residual
+// x - 448 q0 is exact in one fused operation, and q0 + residual * RN(1/448) rounds to the nearest
+// float of the true quotient (448 = 1.75 * 2^8: its reciprocal's rounding error is far from the
+// half-unit cases where this correction can fail).  Infinity and NaN come out as NaN, as the
+// quotients of such a block do anyway.
+__device__ __forceinline__ float div_by_448(float x) {
+  constexpr float r = 1.0f / 448.0f;
+  const float q0 = x * r;
+  return __builtin_fmaf(__builtin_fmaf(-q0, 448.0f, x), r, q0);
+}
 
 // quantises one latent row held as (raw = this lane's 8 NoPE values, rope = lanes 0..7: the RoPE tail) into rec
 __device__ __forceinline__ void quantize_row(const uint4 raw, const uint4 rope, uint8_t* rec, int lane) {
@@ -245,20 +264,20 @@ __device__ __forceinline__ void quantize_row(const uint4 raw, const uint4 rope, 
   amax = fmaxf(amax, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, amax), 0x122, 0xf, 0xf, false)));
   amax = fmaxf(amax, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, amax), 0x124, 0xf, 0xf, false)));
   amax = fmaxf(amax, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, amax), 0x128, 0xf, 0xf, false)));
-  const float scale = __fdiv_rn(fmaxf(amax, 0x1p-126f * 448.0f), 448.0f);
+  const float scale = div_by_448(fmaxf(amax, 0x1p-126f * 448.0f));
   const float r0 = __builtin_amdgcn_rcpf(scale);
   const float inv = __builtin_fmaf(r0, __builtin_fmaf(-scale, r0, 1.0f), r0);    // one Newton step: 1 / scale to one unit
   const float small = scale * 0x1.02p-6f;            // below this a quotient may be an fp8 subnormal
   float qv[8];
-  bool divide = false;
+  uint32_t nearest = 0xffffffffu;                    // smallest distance code of the eight: one compare for all
+  float least = INFINITY;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     qv[i] = v[i] * inv;
-    const uint32_t low = (__float_as_uint(qv[i]) & 0xfffffu) - (0x80000u - 5u);
-    divide |= low <= 10u;
-    divide |= fabsf(v[i]) < small;
+    nearest = min(nearest, (__float_as_uint(qv[i]) - (0x80000u - 5u)) & 0xfffffu);
+    least = fminf(least, fabsf(v[i]));
   }
-  if (divide) {
+  if (nearest <= 10u || least < small) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) qv[i] = __fdiv_rn(v[i], scale);
   }
@@ -301,8 +320,9 @@ __global__ __launch_bounds__(256) void quantize_kernel(const uint16_t* __restric
   }
 #pragma unroll
   for (int j = 0; j < kRowsPerWave; ++j) {
-    if (dst[j] < 0 || dst[j] >= record_rows) continue;           // (wave-uniform)
-    quantize_row(raw[j], rope[j], records + dst[j] * kRowBytesFp8, lane);
+    const int64_t d = wave_uniform(dst[j]);                      // the same in every lane: the record's address is scalar work
+    if (d < 0 || d >= record_rows) continue;
+    quantize_row(raw[j], rope[j], records + d * kRowBytesFp8, lane);
   }
 }
 

@@ -792,6 +792,29 @@ def test_cache_writer_bit_exact(schedule):
         assert np.array_equal(got, want), fmt
 
 
+def test_cache_writer_scale_of_every_block_maximum():
+    """The writer divides a block's maximum by 448 with a multiplication and a fused correction
+    instead of an IEEE division: every positive finite bf16 value is the maximum of one block here
+    (with its half and its negative beside it), and scales and codes must be the oracle's bits."""
+    bits = np.arange(1, 0x7F80, dtype=np.uint16)                         # every positive finite bf16
+    bits = np.concatenate([bits, np.full((-len(bits)) % 4, 0x3F80, np.uint16)])
+    blocks = np.zeros((len(bits), 128), dtype=np.uint16)
+    blocks[:, 17] = bits
+    blocks[:, 90] = bits | 0x8000
+    half = np.where((bits >> 7) > 1, bits - 0x80, 0).astype(np.uint16)   # exponent - 1 where that stays normal
+    blocks[:, 3] = half
+    lat_bits = np.concatenate([blocks.reshape(-1, 512), blocks.reshape(-1, 512)[:, :64]], axis=1)
+    lat = torch.from_numpy(lat_bits.view(np.int16).copy()).view(torch.bfloat16)
+    n = lat.shape[0]
+    cache = torch.zeros((n, 656), dtype=torch.uint8)
+    rc = harness.lib().smla_kv_write(1, lat.data_ptr(), None, cache.data_ptr(), n, n, None)
+    assert rc == 0
+    want = oracle.quantize_kv_records(oracle.bf16_bits_to_f32(lat_bits))
+    got = cache.numpy()
+    assert np.array_equal(got[:, 512:528], want[:, 512:528]), "scales"
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("rows,n,k", [(3, 4096, 2048), (2, 1000, 64), (1, 20000, 300), (2, 70000, 128), (5, 33, 40)])
 def test_topk_indices_exact(rows, n, k):
     g = torch.Generator().manual_seed(rows * 131 + n)
