@@ -220,6 +220,25 @@ def test_quantize_fp8_bit_exact_at_midpoints(dev):
     assert np.array_equal(to_np(ft.quantize_kv_fp8(lat.to(dev))), want)
 
 
+def test_quantize_fp8_scale_of_every_block_maximum(dev):
+    """Every positive finite bf16 value as the maximum of one block (down to the subnormal ones,
+    where the scale is clamped, and just above, where the correction term of the writer's division
+    by 448 is itself subnormal)."""
+    import flagtree_amd as ft
+    bits = np.arange(1, 0x7F80, dtype=np.uint16)
+    bits = np.concatenate([bits, np.full((-len(bits)) % 4, 0x3F80, np.uint16)])
+    blocks = np.zeros((len(bits), 128), dtype=np.uint16)
+    blocks[:, 17] = bits
+    blocks[:, 90] = bits | 0x8000
+    blocks[:, 3] = np.where((bits >> 7) > 1, bits - 0x80, 0).astype(np.uint16)
+    lat_bits = np.concatenate([blocks.reshape(-1, 512), blocks.reshape(-1, 512)[:, :64]], axis=1)
+    lat = torch.from_numpy(lat_bits.view(np.int16).copy()).view(torch.bfloat16)
+    got = to_np(ft.quantize_kv_fp8(lat.to(dev)))
+    want = oracle.quantize_kv_records(oracle.bf16_bits_to_f32(lat_bits))
+    assert np.array_equal(got[:, 512:528], want[:, 512:528]), "scales"
+    assert np.array_equal(got, want)
+
+
 def test_quantize_fp8_bit_exact_random_magnitudes(dev):
     """38 million random quotients over forty decades of block scales."""
     import flagtree_amd as ft
