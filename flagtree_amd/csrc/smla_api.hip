@@ -238,13 +238,14 @@ static int fwd_impl(bool dense, int kv_format, const void* q, const void* kv, co
     p.merge_in_launch = merge_in_launch_ok() ? 1 : 0;
   }
   if (persist_enabled() && device_cus() % 8 == 0) p.persist_workgroups = device_cus();
-  if (n_heads > 32 && head_groups_enabled()) rc = launch_fwd_group(kv_format, p, s);
+  const bool head_groups = n_heads > 32 && head_groups_enabled();    // (that kernel keeps its partial sums as bf16)
+  if (head_groups) rc = launch_fwd_group(kv_format, p, s);
   else if (n_heads > 32) rc = launch_fwd_tall(kv_format, p, s);
   else if (kv_format == SMLA_KV_FP8_B128 && fp8_mfma_enabled()) rc = launch_fwd_few_f8(p, s);
   else if (kv_format == SMLA_KV_FP8_B128 && few_fp8_enabled()) rc = launch_fwd_few_fp8(p, s);
   else rc = launch_fwd_short(kv_format, p, s);
   if (rc != SMLA_OK || n_splits == 1 || p.merge_in_launch) return rc;
-  return launch_merge(p.part_out, p.part_lse, out, lse, n_tokens, n_heads, d_v, n_splits, s);
+  return launch_merge(p.part_out, p.part_lse, out, lse, n_tokens, n_heads, d_v, n_splits, head_groups, s);
 }
 
 int smla_fwd(int kv_format, const void* q, const void* kv, const int32_t* indices,
@@ -313,7 +314,7 @@ int smla_merge_splits(const float* part_out, const float* part_lse, void* out, f
   if (n_tokens <= 0 || n_heads <= 0 || d_v != kDv || (long long)n_tokens * n_heads > 0x7fffffffLL) return SMLA_EINVAL_SHAPE;
   if (n_splits < 1 || n_splits > SMLA_MAX_SPLITS) return SMLA_EINVAL_SPLITS;
   if (!aligned16(part_out) || !aligned16(out)) return SMLA_EINVAL_ALIGN;
-  return launch_merge(part_out, part_lse, out, lse, n_tokens, n_heads, d_v, n_splits,
+  return launch_merge(part_out, part_lse, out, lse, n_tokens, n_heads, d_v, n_splits, false,
                       static_cast<hipStream_t>(stream));
 }
 

@@ -243,7 +243,7 @@ int launch_fwd_group(int kv_format, const Params& p, hipStream_t s);   // n_head
 int launch_fwd_few_fp8(const Params& p, hipStream_t s);                // n_heads <= 32, fp8 records, two workgroups per CU (opt-in)
 int launch_fwd_few_f8(const Params& p, hipStream_t s);                 // n_heads <= 32, fp8 records contracted by fp8 MFMAs, two workgroups per CU (opt-in)
 int launch_merge(const float* part_out, const float* part_lse, void* out, float* lse,
-                 int n_tokens, int n_heads, int d_v, int n_splits, hipStream_t s);
+                 int n_tokens, int n_heads, int d_v, int n_splits, bool partials_bf16, hipStream_t s);
 int launch_gather(const Params& p, int row_bytes, int32_t* phys_out, void* rows_out, hipStream_t s);
 int launch_quantize(const void* src, const int64_t* slot, void* records, int64_t n_rows,
                     int64_t record_rows, hipStream_t s);

@@ -661,6 +661,12 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks,
     *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.out) + ((size_t)t * p.n_heads + head0 + row) * kDv + col8) = w;
   };
   auto lse_index = [&](int ht) { return (size_t)t * p.n_heads + head0 + 16 * ht + l16_e; };
+  // Partial sums of split i of this item, as bf16: [head][512] from head0 on, in the first half of
+  // the area the workspace keeps for fp32 partials.  A normalised partial is an average of cache
+  // values, the output is bf16 anyway, and the merge still weighs and adds in fp32.
+  auto part16 = [&](int i) {
+    return reinterpret_cast<uint16_t*>(p.part_out) + (((size_t)t * p.n_splits + i) * p.n_heads + head0) * kDv;
+  };
   auto head_ok = [&](int ht) { return head0 + 16 * ht + l16_e < p.n_heads; };
 
   const int ns = p.n_splits;
@@ -703,12 +709,15 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks,
         __hip_atomic_store(&p.part_lse[((size_t)t * ns + sp) * p.n_heads + head0 + 16 * ht + l16_e], lse_nat[ht], __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
       stage_tile(ht);
-      float* o = p.part_out + (((size_t)t * ns + sp) * p.n_heads + head0 + 16 * ht) * kDv + col8;
+      // (partials of this kernel are bf16: with four splits of 128 heads the fp32 ones were a third
+      // of the headline decode's traffic, all of it in the tail; see part16)
+      uint16_t* o = part16(sp) + (size_t)(16 * ht) * kDv + col8;
       for (int row = 0; row < 16; ++row) {
         if (16 * ht + row >= n_rows) break;
         const float4 a = staged(row, 0), b = staged(row, 1);
-        hw::store_b128_agent(o + (size_t)row * kDv, f32x4{a.x, a.y, a.z, a.w});
-        hw::store_b128_agent(o + (size_t)row * kDv + 4, f32x4{b.x, b.y, b.z, b.w});
+        hw::u32x4 w;
+        w[0] = pack_bf16(a.x, a.y); w[1] = pack_bf16(a.z, a.w); w[2] = pack_bf16(b.x, b.y); w[3] = pack_bf16(b.z, b.w);
+        hw::store_b128_agent(reinterpret_cast<float*>(o + (size_t)row * kDv), __builtin_bit_cast(f32x4, w));
       }
     }
     hw::wait_vmcnt<0>();
@@ -758,28 +767,26 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks,
           if (q4_e == 0) s_w[wave][b][l16_e] = wi;
         }
         hw::wave_lds_order();
-        f32x4 v[kBatch][kRound][2];
+        hw::u32x4 raw[kBatch][kRound];       // eight bf16 values each; this split's own rows rounded like the others'
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) {
           const int i = i0 + b;
           if (i < ns && i != sp && rows_here > r0) {
-            const hw::buffer_rsrc src = hw::make_rsrc(p.part_out + (((size_t)t * ns + i) * p.n_heads + head0 + 16 * ht) * kDv);
+            const hw::buffer_rsrc src = hw::make_rsrc(part16(i) + (size_t)(16 * ht) * kDv);
 #pragma unroll
             for (int j = 0; j < kRound; ++j) {
-              const uint32_t off = (uint32_t)((min(r0 + j, rows_here - 1) * kDv + col8) * 4);
-              v[b][j][0] = hw::load_b128_agent(src, off);
-              v[b][j][1] = hw::load_b128_agent(src, off + 16);
+              const uint32_t off = (uint32_t)((min(r0 + j, rows_here - 1) * kDv + col8) * 2);
+              raw[b][j] = __builtin_bit_cast(hw::u32x4, hw::load_b128_agent(src, off));
             }
           } else if (i == sp) {
 #pragma unroll
             for (int j = 0; j < kRound; ++j) {
               const float4 a = staged(r0 + j, 0), c = staged(r0 + j, 1);
-              v[b][j][0] = f32x4{a.x, a.y, a.z, a.w};
-              v[b][j][1] = f32x4{c.x, c.y, c.z, c.w};
+              raw[b][j] = hw::u32x4{pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(c.x, c.y), pack_bf16(c.z, c.w)};
             }
           } else {                           // no such split, or rows past the last head: nothing to read, nothing stored
 #pragma unroll
-            for (int j = 0; j < kRound; ++j) { v[b][j][0] = f32x4{0.f, 0.f, 0.f, 0.f}; v[b][j][1] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+            for (int j = 0; j < kRound; ++j) raw[b][j] = hw::u32x4{0u, 0u, 0u, 0u};
           }
         }
 #pragma unroll
@@ -789,9 +796,10 @@ __global__ __launch_bounds__(kNT) void fwd_group_kernel(Params p, int n_hblocks,
             for (int j = 0; j < kRound; ++j) {
               const float rb = s_w[wave][b][r0 + j];
 #pragma unroll
-              for (int c = 0; c < 4; ++c) {
-                sum[j][0][c] = __fadd_rn(sum[j][0][c], __fmul_rn(v[b][j][0][c], rb));
-                sum[j][1][c] = __fadd_rn(sum[j][1][c], __fmul_rn(v[b][j][1][c], rb));
+              for (int c = 0; c < 4; ++c) {   // word c of a row = columns 2c (low half) and 2c + 1
+                const float even = __uint_as_float(raw[b][j][c] << 16), odd = __uint_as_float(raw[b][j][c] & 0xffff0000u);
+                sum[j][c >> 1][2 * (c & 1)] = __fadd_rn(sum[j][c >> 1][2 * (c & 1)], __fmul_rn(even, rb));
+                sum[j][c >> 1][2 * (c & 1) + 1] = __fadd_rn(sum[j][c >> 1][2 * (c & 1) + 1], __fmul_rn(odd, rb));
               }
             }
           }

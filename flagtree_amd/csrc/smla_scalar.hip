@@ -174,6 +174,8 @@ int launch_gather(const Params& p, int row_bytes, int32_t* phys_out, void* rows_
 
 // ---------------------------------------------------------------------------------------
 // merge of split partials: one workgroup of 128 lanes per (token, head); 4 dv columns per lane.
+// (PART16: the partial sums are bf16, packed at the start of the same area: the head-group kernel's)
+template <bool PART16>
 __global__ __launch_bounds__(128) void merge_kernel(const float* __restrict__ part_out,
                                                     const float* __restrict__ part_lse,
                                                     uint16_t* __restrict__ out, float* __restrict__ lse,
@@ -189,8 +191,15 @@ __global__ __launch_bounds__(128) void merge_kernel(const float* __restrict__ pa
     const float w = expf(part_lse[((size_t)t * n_splits + i) * n_heads + h] - m_safe);
     if (w == 0.f) continue;    // also skips partials of empty splits (their out is 0, lse -inf)
     tot += w;
-    const float4 v = reinterpret_cast<const float4*>(
-        part_out + (((size_t)t * n_splits + i) * n_heads + h) * kDv)[threadIdx.x];
+    float4 v;
+    if constexpr (PART16) {
+      const uint2 b = reinterpret_cast<const uint2*>(
+          reinterpret_cast<const uint16_t*>(part_out) + (((size_t)t * n_splits + i) * n_heads + h) * kDv)[threadIdx.x];
+      v = make_float4(__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u), __uint_as_float(b.y << 16),
+                      __uint_as_float(b.y & 0xffff0000u));
+    } else {
+      v = reinterpret_cast<const float4*>(part_out + (((size_t)t * n_splits + i) * n_heads + h) * kDv)[threadIdx.x];
+    }
     acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
   }
   const float inv = tot > 0.f ? 1.f / tot : 0.f;
@@ -202,11 +211,15 @@ __global__ __launch_bounds__(128) void merge_kernel(const float* __restrict__ pa
 }
 
 int launch_merge(const float* part_out, const float* part_lse, void* out, float* lse, int n_tokens,
-                 int n_heads, int d_v, int n_splits, hipStream_t s) {
+                 int n_heads, int d_v, int n_splits, bool partials_bf16, hipStream_t s) {
   if (d_v != kDv) return SMLA_EINVAL_SHAPE;
   dim3 grid((unsigned)n_heads * (unsigned)n_tokens), block(128);
-  hipLaunchKernelGGL(merge_kernel, grid, block, 0, s, part_out, part_lse, static_cast<uint16_t*>(out), lse, n_heads,
-                                      n_splits);
+  if (partials_bf16)
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(merge_kernel<true>), grid, block, 0, s, part_out, part_lse, static_cast<uint16_t*>(out), lse,
+                       n_heads, n_splits);
+  else
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(merge_kernel<false>), grid, block, 0, s, part_out, part_lse, static_cast<uint16_t*>(out), lse,
+                       n_heads, n_splits);
   return hip_status(hipGetLastError());
 }
 
